@@ -1,0 +1,137 @@
+/*
+ * sru_amd: the SRU elementwise recurrence (forward scan and backward scan over
+ * time) as hand-written HIP kernels for gfx950, behind a C ABI.
+ *
+ * These entry points stand where the reference binds its eight TorchScript
+ * operators sru_cuda::sru_[bi_]forward[_simple] and
+ * sru_cuda::sru_[bi_]backward[_simple]
+ * (sru/csrc/sru_cuda_impl.cpp:177-518, registered at :531-546, called from
+ * sru/cuda_functional.py:85-144 and :213-251). One forward and one backward
+ * entry cover all eight: direction count, k, activation, skip type and the
+ * per-step weight_c variant are fields of sru_amd_shape.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless said otherwise; the library never
+ *     allocates, frees or retains memory; the caller owns all buffers;
+ *   - every output cell is written, zeros at padded cells included, so outputs
+ *     may be uninitialised memory (the reference relies on zero-filled
+ *     allocations instead, sru_cuda_impl.cpp:189-190,:225-229);
+ *   - kernels are enqueued on `stream` (a hipStream_t; NULL = the null stream)
+ *     and the call returns without waiting;
+ *   - return value 0 = enqueued, anything else = nothing was launched; no
+ *     exception ever crosses this boundary.
+ *
+ * Layouts (those of the reference)
+ *   U        (L, B, D', k)      k innermost; D' = dirs * hidden
+ *   x, h, c, grad_h, grad_x     (L, B, D')
+ *   weight_c (2, D') float, or, when is_custom, (L, B, D', 2) in `dtype`
+ *   bias     (2, D') float
+ *   c_init, mask_c, c_last, grad_last, grad_init   (B, D') float
+ *   mask_pad (L, B) one byte per cell, non-zero = padded
+ *   scale_x  one float on the device, or NULL for 1
+ * `dtype` is the element type of the large streams U, x, h, c, grad_h, grad_u,
+ * grad_x and of a per-step weight_c / its gradient. The recurrence state and all
+ * arithmetic are float whatever `dtype` is.
+ */
+#ifndef SRU_AMD_H
+#define SRU_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SRU_AMD_ABI_VERSION 1
+
+enum sru_amd_dtype {
+    SRU_AMD_F32 = 0,
+    SRU_AMD_F16 = 1,
+    SRU_AMD_BF16 = 2
+};
+
+enum sru_amd_status {
+    SRU_AMD_OK = 0,
+    SRU_AMD_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+    SRU_AMD_ERR_BAD_SHAPE = 2,      /* a size is <= 0 or the problem exceeds the index range */
+    SRU_AMD_ERR_BAD_FLAGS = 3,      /* dirs, k, activation_type, skip_type, is_custom inconsistent */
+    SRU_AMD_ERR_BAD_DTYPE = 4,
+    SRU_AMD_ERR_MISALIGNED = 5,     /* a stream pointer is not aligned to its element type */
+    SRU_AMD_ERR_WORKSPACE = 6,      /* workspace missing or smaller than required */
+    SRU_AMD_ERR_LAUNCH = 7          /* the HIP runtime refused the launch */
+};
+
+/* Problem description; the fields are the integer arguments of the reference's
+ * general operators (sru/csrc/sru_cuda_impl.cpp:333-347: length, batch_size,
+ * hidden_size, k, activation_type, skip_type, is_custom) plus the direction
+ * count that the reference encodes in the operator name. */
+typedef struct sru_amd_shape {
+    int64_t length;          /* L >= 1 */
+    int64_t batch;           /* B >= 1 */
+    int64_t hidden;          /* d >= 1, per direction */
+    int32_t dirs;            /* 1, or 2: columns with (col % 2d) >= d walk time backwards */
+    int32_t k;               /* 3 or 4 streams per column in U */
+    int32_t activation_type; /* 0 identity, 1 tanh */
+    int32_t skip_type;       /* 0 none; 1 from x (k == 3); 2 from U[..., 3] (k == 4) */
+    int32_t is_custom;       /* 0: weight_c (2, D'); 1: per step (L, B, D', 2) */
+    int32_t dtype;           /* enum sru_amd_dtype */
+} sru_amd_shape;
+
+/* Forward scan. Replaces sru_cuda::sru_forward_simple, sru_bi_forward_simple,
+ * sru_forward and sru_bi_forward (sru/csrc/sru_cuda_impl.cpp:177-207,:255-285,
+ * :333-412) together with the x * scale_x pass and the gather of the last state
+ * that sru/cuda_functional.py:73-78 and :146-153 run around them.
+ *   x        required iff skip_type == 1
+ *   mask_c   NULL = no dropout mask
+ *   mask_pad NULL = no padding
+ *   c        per-step state kept for the backward pass; NULL = do not store it
+ *            (inference)
+ *   c_last   state after the last step of each column's walk: what the
+ *            reference assembles as cat(c[-1, :, :d], c[0, :, d:]) */
+int sru_amd_forward(const sru_amd_shape *shape,
+                    const void *u, const void *x, const void *weight_c,
+                    const float *bias, const float *c_init, const float *mask_c,
+                    const uint8_t *mask_pad, const float *scale_x,
+                    void *h, void *c, float *c_last, void *stream);
+
+/* Bytes of device scratch sru_amd_backward needs for `shape` (0 on a bad
+ * shape). The scratch holds per-column partial sums of the weight_c and bias
+ * gradients between the scan kernel and the batch reduction. */
+size_t sru_amd_backward_workspace_bytes(const sru_amd_shape *shape);
+
+/* Backward scan. Replaces sru_cuda::sru_backward_simple, sru_bi_backward_simple,
+ * sru_backward and sru_bi_backward (sru/csrc/sru_cuda_impl.cpp:210-252,:288-330,
+ * :415-518) together with what sru/cuda_functional.py:204-207 and :253-260 run
+ * around them: the x * scale_x pass, grad_x *= scale_x and the batch sums of
+ * the weight_c / bias gradients.
+ *   c         the per-step state the forward call stored
+ *   grad_x    required iff skip_type == 1; already multiplied by scale_x
+ *   grad_wc   (2, D') float summed over time and batch, or, when is_custom,
+ *             (L, B, D', 2) in `dtype`
+ *   grad_bias (2, D') float summed over time and batch
+ *   workspace device scratch of at least sru_amd_backward_workspace_bytes()
+ *             bytes, 16-byte aligned; contents before and after are undefined
+ * The batch sums are formed in a fixed order: results are bit-reproducible. */
+int sru_amd_backward(const sru_amd_shape *shape,
+                     const void *u, const void *x, const void *weight_c,
+                     const float *bias, const float *c_init, const float *mask_c,
+                     const uint8_t *mask_pad, const float *scale_x,
+                     const void *c, const void *grad_h, const float *grad_last,
+                     void *grad_u, void *grad_x, void *grad_wc, float *grad_bias,
+                     float *grad_init, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
+/* Static, NUL-terminated description of a status code (never NULL). The
+ * reference has no counterpart: its operators throw (sru_cuda_impl_dummy.cpp:19)
+ * or fail inside data_ptr<T>(). */
+const char *sru_amd_status_string(int status);
+
+/* SRU_AMD_ABI_VERSION the library was built with. */
+int sru_amd_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SRU_AMD_H */

@@ -1,0 +1,52 @@
+"""Call sites of the recurrence, mirroring sru/ops.py.
+
+* elementwise_recurrence_gpu   (sru/ops.py:97-142): training entry under autograd.
+* elementwise_recurrence_inference (sru/ops.py:22-94): forward only; here it
+  also skips storing the per-step state, which the reference still writes.
+
+Dtype policy. The reference casts every tensor to float32 unless
+amp_recurrence_fp16 is set and U is float16 (sru/ops.py:116-127), because its
+kernels compute in the tensor dtype. These kernels always compute in float32
+whatever the stream dtype, so the `.float()` copies of U and x are not needed:
+with `native_16bit=True` (default) a float16 / bfloat16 U is read as is and h
+comes back in that dtype; `native_16bit=False` reproduces the reference's
+float32 casts (h is then float32, as in the reference).
+"""
+from typing import List, Optional
+
+import torch
+from torch import Tensor
+
+from .functional import ElementwiseRecurrence, elementwise_recurrence_forward
+
+
+def elementwise_recurrence_gpu(U: Tensor, x: Tensor, weight_c: Tensor, bias: Tensor,
+                               c_init: Tensor, activation_type: int, hidden_size: int,
+                               bidirectional: bool, has_skip_term: bool,
+                               scale_x: Optional[Tensor] = None,
+                               dropout_mask_c: Optional[Tensor] = None,
+                               mask_pad: Optional[Tensor] = None,
+                               amp_recurrence_fp16: bool = False,
+                               native_16bit: bool = True) -> List[Tensor]:
+    if not native_16bit and not (amp_recurrence_fp16 and U.dtype == torch.float16):
+        U, x = U.float(), x.float()
+        if weight_c.dim() > 1:
+            weight_c = weight_c.float()
+    return ElementwiseRecurrence.apply(U, x, weight_c, bias, c_init, activation_type,
+                                       hidden_size, bidirectional, has_skip_term, scale_x,
+                                       dropout_mask_c, mask_pad)
+
+
+def elementwise_recurrence_inference(U: Tensor, x: Tensor, weight_c: Tensor, bias: Tensor,
+                                     c_init: Tensor, activation_type: int, hidden_size: int,
+                                     bidirectional: bool, has_skip_term: bool,
+                                     scale_x: Optional[Tensor] = None,
+                                     dropout_mask_c: Optional[Tensor] = None,
+                                     mask_pad: Optional[Tensor] = None) -> List[Tensor]:
+    # same refusal as sru/ops.py:38
+    assert dropout_mask_c is None, "Dropout mask cannot be set during inference"
+    with torch.no_grad():
+        h, last_hidden, _ = elementwise_recurrence_forward(
+            U, x, weight_c, bias, c_init, activation_type, hidden_size, bidirectional,
+            has_skip_term, scale_x, None, mask_pad, keep_c=False)
+    return h, last_hidden

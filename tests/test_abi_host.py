@@ -1,0 +1,102 @@
+"""CPU-only checks of the boundary: the library loads, exports every symbol the header
+declares, and rejects bad arguments before anything reaches a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from sru_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "sru_amd.h")).read()
+    code = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(sru_amd_[a-z_]+)\s*\(", code))
+    assert declared == set(_lib.SIGNATURES), (declared, set(_lib.SIGNATURES))
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert _lib.load().sru_amd_abi_version() == int(re.search(r"SRU_AMD_ABI_VERSION\s+(\d+)", header).group(1))
+
+
+def test_struct_layout_matches_header():
+    assert ctypes.sizeof(_lib.Shape) == 48
+    assert _lib.Shape.dirs.offset == 24 and _lib.Shape.dtype.offset == 44
+
+
+def _shape(**kw):
+    base = dict(length=4, batch=2, hidden=8, dirs=2, k=3, activation_type=0, skip_type=1,
+                is_custom=0, dtype=0)
+    base.update(kw)
+    return _lib.Shape(*[base[f[0]] for f in _lib.Shape._fields_])
+
+
+FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(length=0), 2), (dict(batch=-1), 2), (dict(hidden=0), 2), (dict(hidden=1 << 31), 2),
+    (dict(length=1 << 60), 2), (dict(dirs=3), 3), (dict(k=5), 3), (dict(k=2), 3),
+    (dict(activation_type=2), 3), (dict(skip_type=3), 3), (dict(skip_type=1, k=4), 3),
+    (dict(skip_type=2, k=3), 3), (dict(is_custom=2), 3), (dict(dtype=7), 4),
+])
+def test_forward_rejects_bad_shapes(kw, code):
+    lib = _lib.load()
+    s = _shape(**kw)
+    assert lib.sru_amd_forward(ctypes.byref(s), *([FAKE] * 11), None) == code
+    assert lib.sru_amd_backward_workspace_bytes(ctypes.byref(s)) == 0
+    assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), 1 << 20, None) == code
+
+
+def test_null_and_misaligned_pointers_and_workspace():
+    lib = _lib.load()
+    s = _shape()
+    assert lib.sru_amd_forward(None, *([FAKE] * 11), None) == 1
+    args = [FAKE] * 11
+    for required in (0, 1, 2, 3, 4, 8, 10):   # u, x (skip from x), weight_c, bias, c_init, h, c_last
+        bad = list(args)
+        bad[required] = None
+        assert lib.sru_amd_forward(ctypes.byref(s), *bad, None) == 1, required
+    odd = ctypes.c_void_p(0x1002)
+    bad = list(args)
+    bad[0] = odd
+    assert lib.sru_amd_forward(ctypes.byref(s), *bad, None) == 5
+    s4 = _shape(k=4, skip_type=2)
+    bad = list(args)
+    bad[0] = ctypes.c_void_p(0x1008)            # k=4 float groups move as 16-byte vectors
+    assert lib.sru_amd_forward(ctypes.byref(s4), *bad, None) == 5
+    need = lib.sru_amd_backward_workspace_bytes(ctypes.byref(s))
+    assert need == 4 * 4 * 2 * 16
+    assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 16), None, need, None) == 6
+    assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), need - 1, None) == 6
+    bad = [FAKE] * 17
+    bad[13] = None                               # grad_x is required when the skip term is x
+    assert lib.sru_amd_backward(ctypes.byref(s), *bad, need, None) == 1
+
+
+def test_status_strings_and_python_error_mapping():
+    for code in range(0, 9):
+        assert _lib.status_string(code)
+    with pytest.raises(ValueError):
+        _lib.check(3, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(7, "x")
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libsru_amd.so"))
+    with pytest.raises(_lib.LibraryError):
+        _lib.load()
+
+
+def test_function_refuses_cpu_tensors():
+    import torch
+    from sru_amd import ElementwiseRecurrence
+    L, B, d = 3, 2, 4
+    with pytest.raises(RuntimeError):
+        ElementwiseRecurrence.apply(torch.randn(L, B, 3 * d), torch.randn(L, B, d), torch.randn(2 * d),
+                                    torch.randn(2 * d), torch.zeros(B, d), 0, d, False, True, None)

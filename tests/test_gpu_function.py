@@ -1,0 +1,88 @@
+"""The autograd boundary on the GPU: sru_amd.ElementwiseRecurrence.apply with the
+reference's argument list (sru/cuda_functional.py:159-167) against the oracle's
+differentiable restatement, in the manner of the reference's own CPU-vs-GPU gradient test
+(test/sru/test_sru.py:128-162; tolerance there 1e-4, here 1e-5)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sru_torch as st
+from tests.cases import Case
+
+pytestmark = pytest.mark.gpu
+
+
+def _apply(fn, c, device, dtype):
+    t = lambda a, rg=True: torch.tensor(a, dtype=dtype, device=device, requires_grad=rg)
+    u, x, wc, bias, c0 = t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0)
+    sx = torch.tensor([c.scale], dtype=dtype, device=device)
+    mc = None if c.mask_c is None else torch.tensor(c.mask_c, dtype=dtype, device=device)
+    pad = None if c.pad is None else torch.tensor(c.pad, device=device)
+    h, last = fn(u, x, wc, bias, c0, c.act, c.d, c.dirs == 2, c.skip_type != 0, sx, mc, pad)
+    gh = torch.tensor(c.gh, dtype=dtype, device=device)
+    gl = torch.tensor(c.gl, dtype=dtype, device=device)
+    ((h * gh).sum() + (last * gl).sum()).backward()
+    grads = [None if v.grad is None else v.grad.double().cpu().numpy() for v in (u, x, wc, bias, c0)]
+    return h.detach().double().cpu().numpy(), last.detach().double().cpu().numpy(), grads
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(L=12, B=3, d=64, dirs=2, pad="right", scale=1.7, mask_c=True),
+    dict(L=9, B=4, d=7, dirs=2, k=4),
+    dict(L=5, B=2, d=3, skip=False),
+    dict(L=6, B=2, d=8, custom=True, act=1),
+    dict(L=3, B=5, d=2, dirs=2),
+])
+def test_function_matches_restatement(cfg):
+    from sru_amd import ElementwiseRecurrence
+    c = Case(seed=41, **cfg).f32()
+    h, last, g = _apply(ElementwiseRecurrence.apply, c, "cuda:0", torch.float32)
+    h_ref, last_ref, g_ref = _apply(st.recurrence, c, "cpu", torch.float64)
+    assert np.abs(h - h_ref).max() <= 1e-5 and np.abs(last - last_ref).max() <= 1e-5
+    for a, b in zip(g, g_ref):
+        if b is None or (c.skip_type != 1 and a is None):
+            continue
+        assert a is not None
+        assert np.abs(a - b).max() <= 1e-5 * max(1.0, np.abs(b).max())
+    if c.skip_type != 1:
+        assert g[1] is None
+
+
+def test_single_step_2d_input_and_inference_entry():
+    from sru_amd import elementwise_recurrence_forward, elementwise_recurrence_inference
+    c = Case(L=1, B=4, d=64, dirs=2, seed=42).f32()
+    dev = "cuda:0"
+    t = lambda a: torch.tensor(a, dtype=torch.float32, device=dev)
+    h, last, cc = elementwise_recurrence_forward(t(c.U[0]), t(c.x[0]), t(c.wc), t(c.bias), t(c.c0),
+                                                 0, c.d, True, True, None)
+    assert h.shape == (4, 128) and cc.shape == (4, 128) and torch.equal(last, cc)
+    h3, last3 = elementwise_recurrence_inference(t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0),
+                                                 0, c.d, True, True, None, None, None)
+    assert torch.equal(h3[0], h) and torch.equal(last3, last)
+    with pytest.raises(AssertionError):
+        elementwise_recurrence_inference(t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0), 0, c.d, True, True,
+                                         None, t(c.c0), None)
+    with pytest.raises(AssertionError):   # mask_pad shape, as sru/cuda_functional.py:70-71
+        elementwise_recurrence_forward(t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0), 0, c.d, True, True,
+                                       None, None, torch.zeros(2, 4, device=dev))
+
+
+def test_amp_style_bf16_streams_against_fp32_run():
+    # U and x arrive in bfloat16 (autocast GEMM output); the reference would cast them to
+    # float32 (sru/ops.py:116-127) and run there. Tolerance: 2e-2 relative to that run.
+    from sru_amd import elementwise_recurrence_gpu
+    c = Case(L=32, B=4, d=128, dirs=2, seed=43, pad="right", scale=1.7)
+    dev = "cuda:0"
+    outs = {}
+    for native in (True, False):
+        t = lambda a, dt=torch.float32: torch.tensor(a, dtype=dt, device=dev, requires_grad=True)
+        u, x = t(c.U, torch.bfloat16), t(c.x, torch.bfloat16)
+        wc, bias, c0 = t(c.wc), t(c.bias), t(c.c0)
+        h, last = elementwise_recurrence_gpu(u, x, wc, bias, c0, 0, c.d, True, True,
+                                             torch.tensor([c.scale], device=dev), None,
+                                             torch.tensor(c.pad, device=dev), native_16bit=native)
+        assert h.dtype == (torch.bfloat16 if native else torch.float32)
+        (h.float() * torch.tensor(c.gh, dtype=torch.float32, device=dev)).sum().backward()
+        outs[native] = [h.float()] + [v.grad.float() for v in (u, x, wc, bias, c0)]
+    for a, b in zip(outs[True], outs[False]):
+        assert float((a - b).abs().max()) <= 2e-2 * max(1.0, float(b.abs().max()))

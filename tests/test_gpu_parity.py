@@ -1,0 +1,138 @@
+"""GPU parity of the HIP kernels, called through the C ABI, against the CPU oracle.
+
+Tolerances (the bar the build is held to):
+  float32 streams : max abs error <= 1e-5 for h, c, c_last, grad_u, grad_x, grad_init
+                    against the float64 oracle on identical inputs; the batch/time-summed
+                    grad_wc and grad_bias are held to 1e-5 * max(1, max|reference|)
+                    (a sum of L*B terms cannot be held to an absolute 1e-5 in float32;
+                    the float32 CPU loop itself does not meet that at the large shapes).
+  float16 / bfloat16 streams : max abs error <= 2e-2 * max(1, max|reference|) against the
+                    float64 oracle fed the same rounded inputs.
+Outputs are pre-filled with NaN: a cell the kernels do not write fails the comparison.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sru_oracle as so
+from tests.abi import DeviceProblem, to_np
+from tests.cases import GRID, Case
+
+pytestmark = pytest.mark.gpu
+
+F32_ABS = 1e-5
+HALF_REL = 2e-2
+
+
+def _err(a, b):
+    assert a.shape == b.shape or a.size == b.size
+    d = np.abs(a.reshape(-1) - b.reshape(-1))
+    assert not np.isnan(d).any(), "unwritten or NaN cells"
+    return float(d.max()) if d.size else 0.0
+
+
+def _scale(ref):
+    return max(1.0, float(np.abs(ref).max()))
+
+
+def check_against_oracle(case, dt="f32", keep_c=True):
+    dp = DeviceProblem(case, dt)
+    rc = dp.rounded_case()
+    h, c, c_last = dp.forward(keep_c=keep_c)
+    h_ref, c_ref, cl_ref = so.forward(*rc.fwd_args(), **rc.kw())
+    tol = (lambda ref: F32_ABS) if dt == "f32" else (lambda ref: HALF_REL * _scale(ref))
+    assert _err(to_np(h), h_ref) <= tol(h_ref)
+    assert _err(to_np(c_last), cl_ref) <= (F32_ABS if dt == "f32" else 1e-3 * _scale(cl_ref))
+    if not keep_c:
+        return
+    assert _err(to_np(c), c_ref) <= tol(c_ref)
+    # backward from the state the device stored (what a training step does)
+    gu, gx, gwc, gb, gi = dp.backward()
+    c_used = to_np(c)
+    g_ref = so.backward(*rc.fwd_args(), c_used, rc.gh, rc.gl, **rc.kw())
+    assert _err(to_np(gu), g_ref[0]) <= tol(g_ref[0])
+    if case.skip_type == 1:
+        assert _err(to_np(gx), g_ref[1]) <= tol(g_ref[1])
+    sum_tol = (lambda ref: F32_ABS * _scale(ref)) if dt == "f32" else (lambda ref: HALF_REL * _scale(ref))
+    assert _err(to_np(gwc), g_ref[2]) <= (tol(g_ref[2]) if case.custom else sum_tol(g_ref[2]))
+    assert _err(to_np(gb), g_ref[3]) <= sum_tol(g_ref[3])
+    assert _err(to_np(gi), g_ref[4]) <= (F32_ABS if dt == "f32" else HALF_REL * _scale(g_ref[4]))
+
+
+_ids = lambda g: "-".join(f"{k}{v}" for k, v in g.items())
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("cfg", GRID, ids=_ids)
+def test_small_grid(cfg, dt):
+    check_against_oracle(Case(seed=21, **cfg), dt)
+
+
+# shapes that exercise whole wavefronts, ragged tails, both loop phases and odd ring fills
+MID = [
+    dict(L=1, B=3, d=64, dirs=2),
+    dict(L=7, B=2, d=128, dirs=2, pad="right", scale=1.7),
+    dict(L=8, B=2, d=64),
+    dict(L=15, B=3, d=64, dirs=2, pad="random", mask_c=True),
+    dict(L=16, B=2, d=96, dirs=2, k=4, pad="right"),
+    dict(L=17, B=5, d=50, dirs=2, scale=1.3, pad="right"),
+    dict(L=33, B=4, d=192, k=4),
+    dict(L=40, B=3, d=130, pad="random"),
+    dict(L=64, B=8, d=256, dirs=2, pad="right", scale=1.7, mask_c=True),
+    dict(L=25, B=2, d=64, dirs=2, custom=True, pad="right"),
+    dict(L=25, B=2, d=64, dirs=2, act=1, k=4),
+    dict(L=25, B=2, d=64, skip=False, pad="random"),
+]
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("cfg", MID, ids=_ids)
+def test_mid_shapes(cfg, dt):
+    check_against_oracle(Case(seed=22, **cfg), dt)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+def test_inference_variant_without_state_store(dt):
+    check_against_oracle(Case(L=40, B=4, d=128, dirs=2, seed=23, pad="right", scale=1.7), dt, keep_c=False)
+    check_against_oracle(Case(L=9, B=2, d=5, dirs=2, k=4, seed=23), dt, keep_c=False)
+
+
+def test_reference_config_1_readme_example_layer():
+    # 2-layer uni SRU, input=hidden=128, L=20, B=32, highway_bias=-2 (README.md example)
+    c = Case(L=20, B=32, d=128, seed=31, zero_c0=True, gate_bias=-2.0)
+    check_against_oracle(c.f32(), "f32")
+
+
+def test_reference_config_2_shape_with_lengths():
+    # bi d=512, L=128, B=32, right-padded lengths; layer 0 is k=4, the others k=3
+    check_against_oracle(Case(L=128, B=32, d=512, dirs=2, k=4, seed=32, pad="right", zero_c0=True).f32())
+    check_against_oracle(Case(L=128, B=32, d=512, dirs=2, k=3, seed=33, pad="right", zero_c0=True).f32())
+
+
+def test_padded_cells_cannot_leak_bit_identical():
+    # misc/test_sru.py:34-42 at kernel level, forward and backward
+    c = Case(L=24, B=4, d=128, dirs=2, seed=34, pad="random", mask_c=True, scale=1.7)
+    a = DeviceProblem(c)
+    out_a = [t.clone() for t in a.forward()] + [t.clone() for t in a.backward()]
+    c2 = Case(L=24, B=4, d=128, dirs=2, seed=34, pad="random", mask_c=True, scale=1.7)
+    c2.U[c2.pad] = np.nan
+    c2.x[c2.pad] = 1e30
+    c2.gh[c2.pad] = np.inf
+    b = DeviceProblem(c2)
+    out_b = list(b.forward()) + list(b.backward())
+    for p, q in zip(out_a, out_b):
+        assert torch.equal(p, q)
+    pad = torch.tensor(c.pad, device="cuda:0")
+    assert float(out_a[0][pad].abs().max()) == 0.0      # h
+    assert float(out_a[3][pad].abs().max()) == 0.0      # grad_u
+    assert float(out_a[4][pad].abs().max()) == 0.0      # grad_x
+
+
+def test_backward_is_bit_reproducible():
+    c = Case(L=50, B=16, d=256, dirs=2, seed=35, pad="right")
+    a = DeviceProblem(c)
+    a.forward()
+    first = [t.clone() for t in a.backward()]
+    for _ in range(3):
+        again = a.backward()
+        assert all(torch.equal(p, q) for p, q in zip(first, again))
