@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the SRU recurrence hot path on one MI355X.
+
+A step = one forward scan + one backward scan of ONE layer's recurrence, called
+through the C ABI (include/sru_amd.h) on synthetic inputs already resident in HBM.
+Workload = the headline configuration: bidirectional, d=1024 per direction
+(D'=2048), L=256, B=64, k=3 with the skip term read from x, scale_x=sqrt(3), c0=0,
+float32 streams. Inputs rotate over several buffer sets so that no step finds its
+operands in the last-level cache.
+
+Prints ONE JSON line: tokens/s (tokens = L*B per step), per-kernel HIP-event timings,
+the HBM roofline of the dominant kernel (the backward scan) on algorithmic bytes, and
+a single-core CPU baseline timed on this host with the CPU oracle (reported only).
+"""
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+WORKLOADS = {
+    # name: L, B, d, dirs, k
+    "bi-SRU d=1024 L=256 B=64 fp32 k=3": (256, 64, 1024, 2, 3),
+}
+DT_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
+
+
+def cpu_baseline(L, B, d, dirs, k, budget_s=12.0):
+    """Times the float32 CPU oracle (serial loop, 1 core) on a slice of the batch."""
+    from oracle import sru_oracle as so
+    Bc = B
+    Dp = d * dirs
+    rng = np.random.default_rng(0)
+    U = rng.standard_normal((L, Bc, Dp * k), dtype=np.float32)
+    x = rng.standard_normal((L, Bc, Dp), dtype=np.float32)
+    wc = rng.uniform(-1.2, 1.2, 2 * Dp).astype(np.float32)
+    bias = np.zeros(2 * Dp, np.float32)
+    c0 = np.zeros((Bc, Dp), np.float32)
+    gh = rng.standard_normal((L, Bc, Dp), dtype=np.float32)
+    gl = np.zeros((Bc, Dp), np.float32)
+    kw = dict(d=d, dirs=dirs, k=k, skip_type=1 if k == 3 else 2, scale_x=3 ** 0.5, precision="f32")
+    so.lib()
+    reps, spent = 0, 0.0
+    while reps < 1 or spent < budget_s:
+        t0 = time.perf_counter()
+        _, c_all, _ = so.forward(U, x, wc, bias, c0, **kw)
+        so.backward(U, x, wc, bias, c0, c_all, gh, gl, **kw)
+        spent += time.perf_counter() - t0
+        reps += 1
+    tokens = L * Bc * reps
+    return {"value": tokens / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"{reps} x (forward+backward) of the same layer at batch {Bc} of {B} "
+                      f"(L={L}, D'={Dp}, k={k}, float32 serial C loop), {spent:.1f} s",
+            "host_cores": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--dtype", default="f32", choices=sorted(DT_BYTES))
+    ap.add_argument("--sets", type=int, default=4, help="rotating buffer sets")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also time a plain device copy of 1 GiB (context for the roofline figures "
+                         "and the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures the recurrence on ONE GPU only "
+                 "(columns are independent; no multi-GPU path exists): run with --gpus 1")
+
+    import torch
+    from sru_amd import _lib
+    from tests.abi import TORCH_DT, CODE, p
+
+    name = next(iter(WORKLOADS))
+    L, B, d, dirs, k = WORKLOADS[name]
+    Dp = d * dirs
+    ncols, cells = B * Dp, L * B * Dp
+    dev = torch.device("cuda:0")
+    tdt = TORCH_DT[args.dtype]
+    es = DT_BYTES[args.dtype]
+    lib = _lib.load()
+    shape = _lib.Shape(L, B, d, dirs, k, 0, 1 if k == 3 else 2, 0, CODE[args.dtype])
+
+    g = torch.Generator(device=dev).manual_seed(1234)
+    sets = []
+    for _ in range(args.sets):
+        s = dict(
+            U=torch.randn(L, B, Dp * k, device=dev, generator=g).to(tdt),
+            x=torch.randn(L, B, Dp, device=dev, generator=g).to(tdt),
+            gh=torch.randn(L, B, Dp, device=dev, generator=g).to(tdt),
+            h=torch.empty(L, B, Dp, device=dev, dtype=tdt),
+            c=torch.empty(L, B, Dp, device=dev, dtype=tdt),
+            gu=torch.empty(L, B, Dp * k, device=dev, dtype=tdt),
+            gx=torch.empty(L, B, Dp, device=dev, dtype=tdt),
+        )
+        sets.append(s)
+    wc = (torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1) * 1.5 ** 0.5
+    bias = torch.zeros(2 * Dp, device=dev)
+    c0 = torch.zeros(B, Dp, device=dev)
+    gl = torch.zeros(B, Dp, device=dev)
+    scale = torch.tensor([3 ** 0.5], device=dev)
+    c_last = torch.empty(B, Dp, device=dev)
+    gwc = torch.empty(2 * Dp, device=dev)
+    gb = torch.empty(2 * Dp, device=dev)
+    gi = torch.empty(B, Dp, device=dev)
+    ws_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(shape))
+    ws = torch.empty(ws_bytes // 4, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+    def fwd(s):
+        rc = lib.sru_amd_forward(ctypes.byref(shape), p(s["U"]), p(s["x"]), p(wc), p(bias), p(c0), None,
+                                 None, p(scale), p(s["h"]), p(s["c"]), p(c_last), stream)
+        assert rc == 0, _lib.status_string(rc)
+
+    def bwd(s):
+        rc = lib.sru_amd_backward(ctypes.byref(shape), p(s["U"]), p(s["x"]), p(wc), p(bias), p(c0), None,
+                                  None, p(scale), p(s["c"]), p(s["gh"]), p(gl), p(s["gu"]), p(s["gx"]),
+                                  p(gwc), p(gb), p(gi), p(ws), ctypes.c_size_t(ws_bytes), stream)
+        assert rc == 0, _lib.status_string(rc)
+
+    copy_cal = None
+    if args.calibrate_copy:
+        n = 1 << 28                                    # 2^28 floats = 1 GiB read + 1 GiB written
+        src = torch.randn(n, device=dev)
+        dst = torch.empty_like(src)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        dst.copy_(src)
+        e0.record()
+        for _ in range(5):
+            dst.copy_(src)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 5
+        copy_cal = {"bytes_read": 4 * n, "bytes_written": 4 * n, "avg_us": us,
+                    "GBps": 8 * n / (us * 1e-6) / 1e9, "frac_of_hbm_peak": 8 * n / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+        del src, dst
+
+    for i in range(args.warmup):
+        fwd(sets[i % args.sets])
+        bwd(sets[i % args.sets])
+    # events live on the stream the kernels are launched on (torch's current stream)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        s = sets[i % args.sets]
+        ev[i][0].record()
+        fwd(s)
+        ev[i][1].record()
+        bwd(s)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    ms_step = (t1 - t0) * 1e3 / args.steps
+    fwd_us = 1e3 * sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_us = 1e3 * sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    traffic = None   # HBM bytes per backward launch from the committed rocprofv3 counter runs
+    tfile = os.path.join(ROOT, "profiles", "traffic_bi_d1024_L256_B64_%s.json" % args.dtype)
+    if os.path.exists(tfile):
+        traffic = json.load(open(tfile))["backward_scan"]["traffic_bytes"]
+    fwd_bytes = 6 * es * cells     # reads U (k) and x, writes h and c
+    bwd_bytes = 10 * es * cells    # reads U (k), x, c, grad_h; writes grad_u (k), grad_x
+    bwd_gbs = bwd_bytes / (bwd_us * 1e-6) / 1e9
+    out = {
+        "metric": "recurrence tokens/sec & HBM GB/s (%peak), bi-SRU d=1024 L=256 B=64",
+        "value": L * B / (ms_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": name, "length": L, "batch": B, "hidden_per_direction": d,
+                   "directions": dirs, "k": k, "pass": "forward+backward, one layer",
+                   "buffer_sets": args.sets},
+        "roofline": {"bound": "hbm", "kernel": "backward_scan (+ reduce_partials)",
+                     "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "algorithmic_bytes_per_launch": bwd_bytes, "avg_us": bwd_us},
+        "kernels": {
+            "forward_scan": {"avg_us": fwd_us, "algorithmic_GBps": fwd_bytes / (fwd_us * 1e-6) / 1e9,
+                             "frac_of_hbm_peak": fwd_bytes / (fwd_us * 1e-6) / 1e9 / HBM_PEAK_GBS},
+            "backward_scan+reduce": {"avg_us": bwd_us, "algorithmic_GBps": bwd_gbs,
+                                     "frac_of_hbm_peak": bwd_gbs / HBM_PEAK_GBS},
+            "forward+backward": {"avg_us": fwd_us + bwd_us,
+                                 "algorithmic_GBps": (fwd_bytes + bwd_bytes) / ((fwd_us + bwd_us) * 1e-6) / 1e9,
+                                 "frac_of_hbm_peak": (fwd_bytes + bwd_bytes) / ((fwd_us + bwd_us) * 1e-6) / 1e9 / HBM_PEAK_GBS},
+        },
+    }
+    if copy_cal is not None:
+        out["copy_calibration"] = copy_cal
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(L, B, d, dirs, k)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -393,9 +393,10 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
 
 // ================================================================= batch reduction
 // partial (4, B, D') -> grad_wc (2, D'), grad_bias (2, D'). One workgroup per 64 hidden
-// indices and per quantity; 4 wavefronts split the batch, accumulate in double and are
-// combined through LDS in a fixed order, so the result does not depend on scheduling.
-constexpr int kReduceSlices = 4;
+// indices and per quantity; its 16 wavefronts take every 16th batch row each (loads of
+// a wavefront are 256 contiguous bytes), accumulate in double and are combined through
+// LDS in a fixed order, so the result does not depend on scheduling.
+constexpr int kReduceSlices = 16;
 
 __global__ void __launch_bounds__(64 * kReduceSlices)
 reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t B, int32_t Dp) {
@@ -407,7 +408,16 @@ reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t 
     double sum = 0.0;
     if (j < Dp) {
         const float *src = partial + ((int64_t)q * B) * Dp + j;
-        for (int64_t b = slice; b < B; b += kReduceSlices) sum += (double)src[b * Dp];
+        int64_t b = slice;
+        for (; b + 3 * kReduceSlices < B; b += 4 * kReduceSlices) {  // 4 loads in flight
+            const float v0 = src[b * Dp], v1 = src[(b + kReduceSlices) * Dp];
+            const float v2 = src[(b + 2 * kReduceSlices) * Dp], v3 = src[(b + 3 * kReduceSlices) * Dp];
+            sum += (double)v0;
+            sum += (double)v1;
+            sum += (double)v2;
+            sum += (double)v3;
+        }
+        for (; b < B; b += kReduceSlices) sum += (double)src[b * Dp];
     }
     acc[slice][lane] = sum;
     __syncthreads();
