@@ -27,8 +27,14 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 WORKLOADS = {
-    # name: L, B, d, dirs, k
-    "bi-SRU d=1024 L=256 B=64 fp32 k=3": (256, 64, 1024, 2, 3),
+    # key: (name, L, B, d, dirs, k, forward_only, padded). "headline" is the configuration the
+    # metric is quoted on; the others are the reference's remaining GPU configurations at
+    # one layer, kept for side measurements (--workload).
+    "headline": ("bi-SRU d=1024 L=256 B=64 k=3", 256, 64, 1024, 2, 3, False, False),
+    "headline-k4": ("bi-SRU d=1024 L=256 B=64 k=4", 256, 64, 1024, 2, 4, False, False),
+    "config2": ("bi-SRU d=512 L=128 B=32 k=3, right-padded lengths in [32,128]", 128, 32, 512, 2, 3, False, True),
+    "config4": ("uni-SRU d=2048 L=512 B=16 k=3", 512, 16, 2048, 1, 3, False, False),
+    "config5": ("bi-SRU d=256 L=4096 B=256 k=3 forward only, lengths in [1024,4096]", 4096, 256, 256, 2, 3, True, True),
 }
 DT_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
 
@@ -69,6 +75,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--dtype", default="f32", choices=sorted(DT_BYTES))
     ap.add_argument("--sets", type=int, default=4, help="rotating buffer sets")
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "
@@ -82,8 +89,8 @@ def main():
     from sru_amd import _lib
     from tests.abi import TORCH_DT, CODE, p
 
-    name = next(iter(WORKLOADS))
-    L, B, d, dirs, k = WORKLOADS[name]
+    name, L, B, d, dirs, k, fwd_only, padded = WORKLOADS[args.workload]
+    name += " " + args.dtype
     Dp = d * dirs
     ncols, cells = B * Dp, L * B * Dp
     dev = torch.device("cuda:0")
@@ -111,6 +118,10 @@ def main():
     gl = torch.zeros(B, Dp, device=dev)
     scale = torch.tensor([3 ** 0.5], device=dev)
     c_last = torch.empty(B, Dp, device=dev)
+    pad = None
+    if padded:
+        lens = torch.randint(L // 4, L + 1, (B,), device=dev, generator=g)
+        pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :]).view(torch.uint8).contiguous()
     gwc = torch.empty(2 * Dp, device=dev)
     gb = torch.empty(2 * Dp, device=dev)
     gi = torch.empty(B, Dp, device=dev)
@@ -119,13 +130,17 @@ def main():
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
     def fwd(s):
-        rc = lib.sru_amd_forward(ctypes.byref(shape), p(s["U"]), p(s["x"]), p(wc), p(bias), p(c0), None,
-                                 None, p(scale), p(s["h"]), p(s["c"]), p(c_last), stream)
+        rc = lib.sru_amd_forward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if k == 3 else None, p(wc), p(bias),
+                                 p(c0), None, p(pad), p(scale) if k == 3 else None, p(s["h"]),
+                                 None if fwd_only else p(s["c"]), p(c_last), stream)
         assert rc == 0, _lib.status_string(rc)
 
     def bwd(s):
-        rc = lib.sru_amd_backward(ctypes.byref(shape), p(s["U"]), p(s["x"]), p(wc), p(bias), p(c0), None,
-                                  None, p(scale), p(s["c"]), p(s["gh"]), p(gl), p(s["gu"]), p(s["gx"]),
+        if fwd_only:
+            return
+        rc = lib.sru_amd_backward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if k == 3 else None, p(wc), p(bias),
+                                  p(c0), None, p(pad), p(scale) if k == 3 else None, p(s["c"]), p(s["gh"]),
+                                  p(gl), p(s["gu"]), p(s["gx"]) if k == 3 else None,
                                   p(gwc), p(gb), p(gi), p(ws), ctypes.c_size_t(ws_bytes), stream)
         assert rc == 0, _lib.status_string(rc)
 
@@ -168,10 +183,12 @@ def main():
     bwd_us = 1e3 * sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
     traffic = None   # HBM bytes per backward launch from the committed rocprofv3 counter runs
     tfile = os.path.join(ROOT, "profiles", "traffic_bi_d1024_L256_B64_%s.json" % args.dtype)
-    if os.path.exists(tfile):
+    if args.workload == "headline" and os.path.exists(tfile):
         traffic = json.load(open(tfile))["backward_scan"]["traffic_bytes"]
-    fwd_bytes = 6 * es * cells     # reads U (k) and x, writes h and c
-    bwd_bytes = 10 * es * cells    # reads U (k), x, c, grad_h; writes grad_u (k), grad_x
+    fwd_bytes = (5 if fwd_only else 6) * es * cells   # reads U (k) and x (k=3), writes h and (training) c
+    bwd_bytes = 10 * es * cells    # reads U (k), x (k=3), c, grad_h; writes grad_u (k), grad_x (k=3)
+    if fwd_only:
+        bwd_us = float("nan")
     bwd_gbs = bwd_bytes / (bwd_us * 1e-6) / 1e9
     out = {
         "metric": "recurrence tokens/sec & HBM GB/s (%peak), bi-SRU d=1024 L=256 B=64",
@@ -201,6 +218,13 @@ def main():
         out["copy_calibration"] = copy_cal
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(L, B, d, dirs, k)
+    if fwd_only:   # side measurement: the forward scan is the only kernel
+        out["roofline"].update(kernel="forward_scan (inference, no state store)",
+                               achieved=out["kernels"]["forward_scan"]["algorithmic_GBps"],
+                               frac=out["kernels"]["forward_scan"]["frac_of_hbm_peak"],
+                               algorithmic_bytes_per_launch=fwd_bytes, avg_us=fwd_us)
+        for key in ("backward_scan+reduce", "forward+backward"):
+            out["kernels"].pop(key)
     print(json.dumps(out), flush=True)
 
 

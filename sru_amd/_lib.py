@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libsru_amd.so")
+# SRU_AMD_LIBRARY points at another build of the same library (tuning builds)
+LIB_PATH = os.environ.get("SRU_AMD_LIBRARY") or os.path.join(_HERE, "libsru_amd.so")
 ABI_VERSION = 1
 
 F32, F16, BF16 = 0, 1, 2

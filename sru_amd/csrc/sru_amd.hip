@@ -5,10 +5,8 @@
 
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
-#include <type_traits>
-
-#include "sru_scan.h"
+#include "sru_launch.h"
+#include "sru_reduce.h"
 
 namespace {
 
@@ -41,86 +39,6 @@ int check_shape(const sru_amd_shape *s) {
     const int64_t ncols = s->batch * Dp;
     if (s->length > (INT64_C(1) << 56) / (ncols * 4)) return SRU_AMD_ERR_BAD_SHAPE;
     return SRU_AMD_OK;
-}
-
-int ring_depth(const char *var, int fallback) {
-    const char *e = std::getenv(var);
-    if (!e) return fallback;
-    const int v = std::atoi(e);
-    return (v == 4 || v == 8 || v == 12 || v == 16) ? v : fallback;
-}
-
-// Fast kernels exist for the two layouts the SRU layer produces with a skip term and no
-// tanh / per-step weight_c: (k=3, skip from x) and (k=4, skip from U[..., 3]); whether a
-// padding mask is given and whether c is stored are compiled in. Everything else runs
-// the general kernels. Only the float (k=3, skip from x) fast kernels are built at more
-// than one ring depth.
-template <typename T, int K, int SKIP, int MODE>
-void launch_forward(const FwdParams &p, dim3 grid, hipStream_t st, int depth) {
-    if constexpr (std::is_same<T, float>::value && K == 3 && !(MODE & kGeneral)) {
-        switch (depth) {
-        case 4: hipLaunchKernelGGL((forward_scan<T, K, SKIP, MODE, 4>), grid, dim3(kBlock), 0, st, p); return;
-        case 12: hipLaunchKernelGGL((forward_scan<T, K, SKIP, MODE, 12>), grid, dim3(kBlock), 0, st, p); return;
-        case 16: hipLaunchKernelGGL((forward_scan<T, K, SKIP, MODE, 16>), grid, dim3(kBlock), 0, st, p); return;
-        default: break;
-        }
-    }
-    hipLaunchKernelGGL((forward_scan<T, K, SKIP, MODE, 8>), grid, dim3(kBlock), 0, st, p);
-}
-
-template <typename T, int K, int SKIP, int MODE>
-void launch_backward(const BwdParams &p, dim3 grid, hipStream_t st, int depth) {
-    if constexpr (std::is_same<T, float>::value && K == 3 && !(MODE & kGeneral)) {
-        switch (depth) {
-        case 4: hipLaunchKernelGGL((backward_scan<T, K, SKIP, MODE, 4>), grid, dim3(kBlock), 0, st, p); return;
-        case 12: hipLaunchKernelGGL((backward_scan<T, K, SKIP, MODE, 12>), grid, dim3(kBlock), 0, st, p); return;
-        case 16: hipLaunchKernelGGL((backward_scan<T, K, SKIP, MODE, 16>), grid, dim3(kBlock), 0, st, p); return;
-        default: break;
-        }
-    }
-    hipLaunchKernelGGL((backward_scan<T, K, SKIP, MODE, 8>), grid, dim3(kBlock), 0, st, p);
-}
-
-template <typename T, int K, int SKIP>
-void fast_forward(const FwdParams &p, dim3 grid, hipStream_t st, int depth) {
-    const int mode = (p.pad ? kHasPad : 0) | (p.c ? kKeepC : 0);
-    switch (mode) {
-    case 0: launch_forward<T, K, SKIP, 0>(p, grid, st, depth); break;
-    case kHasPad: launch_forward<T, K, SKIP, kHasPad>(p, grid, st, depth); break;
-    case kKeepC: launch_forward<T, K, SKIP, kKeepC>(p, grid, st, depth); break;
-    default: launch_forward<T, K, SKIP, kHasPad | kKeepC>(p, grid, st, depth); break;
-    }
-}
-
-template <typename T, int K, int SKIP>
-void fast_backward(const BwdParams &p, dim3 grid, hipStream_t st, int depth) {
-    if (p.pad) launch_backward<T, K, SKIP, kHasPad>(p, grid, st, depth);
-    else launch_backward<T, K, SKIP, 0>(p, grid, st, depth);
-}
-
-// (k, skip_type) pairs that pass check_shape: (3,0) (3,1) (4,0) (4,2).
-template <typename T>
-void dispatch_forward(const sru_amd_shape &s, const FwdParams &p, dim3 grid, hipStream_t st, int depth) {
-    const bool general = s.activation_type != 0 || s.is_custom != 0 || s.skip_type == 0;
-    if (!general) {
-        if (s.k == 3) fast_forward<T, 3, 1>(p, grid, st, depth);
-        else fast_forward<T, 4, 2>(p, grid, st, depth);
-    } else if (s.k == 3 && s.skip_type == 1) launch_forward<T, 3, 1, kGeneral>(p, grid, st, 8);
-    else if (s.k == 3) launch_forward<T, 3, 0, kGeneral>(p, grid, st, 8);
-    else if (s.skip_type == 2) launch_forward<T, 4, 2, kGeneral>(p, grid, st, 8);
-    else launch_forward<T, 4, 0, kGeneral>(p, grid, st, 8);
-}
-
-template <typename T>
-void dispatch_backward(const sru_amd_shape &s, const BwdParams &p, dim3 grid, hipStream_t st, int depth) {
-    const bool general = s.activation_type != 0 || s.is_custom != 0 || s.skip_type == 0;
-    if (!general) {
-        if (s.k == 3) fast_backward<T, 3, 1>(p, grid, st, depth);
-        else fast_backward<T, 4, 2>(p, grid, st, depth);
-    } else if (s.k == 3 && s.skip_type == 1) launch_backward<T, 3, 1, kGeneral>(p, grid, st, 8);
-    else if (s.k == 3) launch_backward<T, 3, 0, kGeneral>(p, grid, st, 8);
-    else if (s.skip_type == 2) launch_backward<T, 4, 2, kGeneral>(p, grid, st, 8);
-    else launch_backward<T, 4, 0, kGeneral>(p, grid, st, 8);
 }
 
 }  // namespace
@@ -165,13 +83,11 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
     p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
     p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
 
-    const dim3 grid((unsigned)((p.ncols + kBlock - 1) / kBlock));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int depth = ring_depth("SRU_AMD_FWD_DEPTH", 8);
     (void)hipGetLastError();
-    if (s.dtype == SRU_AMD_F32) dispatch_forward<float>(s, p, grid, st, depth);
-    else if (s.dtype == SRU_AMD_F16) dispatch_forward<half_bits>(s, p, grid, st, depth);
-    else dispatch_forward<bf16_bits>(s, p, grid, st, depth);
+    if (s.dtype == SRU_AMD_F32) launch_forward<float>(s, p, st);
+    else if (s.dtype == SRU_AMD_F16) launch_forward<half_bits>(s, p, st);
+    else launch_forward<bf16_bits>(s, p, st);
     return hipGetLastError() == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
 }
 
@@ -212,13 +128,11 @@ int sru_amd_backward(const sru_amd_shape *shape, const void *u, const void *x, c
     p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
     p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
 
-    const dim3 grid((unsigned)((p.ncols + kBlock - 1) / kBlock));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int depth = ring_depth("SRU_AMD_BWD_DEPTH", 8);
     (void)hipGetLastError();
-    if (s.dtype == SRU_AMD_F32) dispatch_backward<float>(s, p, grid, st, depth);
-    else if (s.dtype == SRU_AMD_F16) dispatch_backward<half_bits>(s, p, grid, st, depth);
-    else dispatch_backward<bf16_bits>(s, p, grid, st, depth);
+    if (s.dtype == SRU_AMD_F32) launch_backward<float>(s, p, st);
+    else if (s.dtype == SRU_AMD_F16) launch_backward<half_bits>(s, p, st);
+    else launch_backward<bf16_bits>(s, p, st);
     if (hipGetLastError() != hipSuccess) return SRU_AMD_ERR_LAUNCH;
 
     const dim3 rgrid((unsigned)((p.Dp + 63) / 64), 4);

@@ -1,0 +1,140 @@
+// Kernel selection for one stream element type T. Included by scan_<type>.hip only.
+//
+// Fast kernels exist for the two layouts the SRU layer produces with a skip term and no
+// tanh / per-step weight_c: (k=3, skip from x) and (k=4, skip from U[..., 3]); whether a
+// padding mask is given and whether c is stored are compiled in. Everything else (tanh,
+// per-step weight_c, no skip term) runs the general kernels, one column per lane.
+#pragma once
+
+#include "sru_launch.h"
+
+namespace sru_amd {
+
+// Columns per lane and ring depths of the fast kernels, per element type (the macros let
+// a tuning build override them from the compiler command line).
+#ifndef SRU_AMD_F32_COLS
+#define SRU_AMD_F32_COLS 1
+#endif
+#ifndef SRU_AMD_F32_FWD_DEPTH
+#define SRU_AMD_F32_FWD_DEPTH 8
+#endif
+#ifndef SRU_AMD_F32_BWD_DEPTH
+#define SRU_AMD_F32_BWD_DEPTH 8
+#endif
+#ifndef SRU_AMD_H16_FWD_DEPTH
+#define SRU_AMD_H16_FWD_DEPTH 8
+#endif
+#ifndef SRU_AMD_H16_BWD_DEPTH
+#define SRU_AMD_H16_BWD_DEPTH 8
+#endif
+template <typename T> struct Tune;
+template <> struct Tune<float> {
+    static constexpr int kCols = SRU_AMD_F32_COLS, kFwdDepth = SRU_AMD_F32_FWD_DEPTH,
+                         kBwdDepth = SRU_AMD_F32_BWD_DEPTH;
+};
+template <> struct Tune<half_bits> {
+    static constexpr int kCols = 2, kFwdDepth = SRU_AMD_H16_FWD_DEPTH, kBwdDepth = SRU_AMD_H16_BWD_DEPTH;
+};
+template <> struct Tune<bf16_bits> {
+    static constexpr int kCols = 2, kFwdDepth = SRU_AMD_H16_FWD_DEPTH, kBwdDepth = SRU_AMD_H16_BWD_DEPTH;
+};
+constexpr int kGeneralDepth = 8;
+
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+inline dim3 grid_for(int64_t ncols, int cols) {
+    const int64_t lanes = ncols / cols;
+    return dim3((unsigned)((lanes + kBlock - 1) / kBlock));
+}
+
+// Two columns per lane need an even d (a pair must not straddle a direction or a batch
+// row) and stream pointers aligned to the pair groups.
+template <typename T, int K>
+bool pair_ok(const sru_amd_shape &s, std::initializer_list<const void *> wide,
+             std::initializer_list<const void *> narrow) {
+    if (Tune<T>::kCols != 2 || (s.hidden % 2) != 0) return false;
+    const size_t es = sizeof(T);
+    for (const void *q : wide)
+        if (q && !aligned_to(q, group_align((int)(2 * K * es)))) return false;
+    for (const void *q : narrow)
+        if (q && !aligned_to(q, group_align((int)(2 * es)))) return false;
+    return true;
+}
+
+template <typename T, int K, int SKIP, int COLS>
+void fast_forward(const FwdParams &p, hipStream_t st) {
+    constexpr int P = Tune<T>::kFwdDepth;
+    const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
+    const int mode = (p.pad ? kHasPad : 0) | (p.c ? kKeepC : 0);
+    switch (mode) {
+    case 0: hipLaunchKernelGGL((forward_scan<T, K, SKIP, 0, COLS, P>), grid, block, 0, st, p); break;
+    case kHasPad: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad, COLS, P>), grid, block, 0, st, p); break;
+    case kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kKeepC, COLS, P>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kKeepC, COLS, P>), grid, block, 0, st, p); break;
+    }
+}
+
+template <typename T, int K, int SKIP, int COLS>
+void fast_backward(const BwdParams &p, hipStream_t st) {
+    constexpr int P = Tune<T>::kBwdDepth;
+    const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
+    if (p.pad) hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad, COLS, P>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((backward_scan<T, K, SKIP, 0, COLS, P>), grid, block, 0, st, p);
+}
+
+template <typename T, int K, int SKIP>
+void pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
+    if constexpr (Tune<T>::kCols == 2) {
+        if (pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c})) return fast_forward<T, K, SKIP, 2>(p, st);
+    }
+    fast_forward<T, K, SKIP, 1>(p, st);
+}
+
+template <typename T, int K, int SKIP>
+void pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
+    if constexpr (Tune<T>::kCols == 2) {
+        if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) return fast_backward<T, K, SKIP, 2>(p, st);
+    }
+    fast_backward<T, K, SKIP, 1>(p, st);
+}
+
+// (k, skip_type) pairs that pass the shape check: (3,0) (3,1) (4,0) (4,2).
+template <typename T>
+void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
+    const bool general = s.activation_type != 0 || s.is_custom != 0 || s.skip_type == 0;
+    const dim3 grid = grid_for(p.ncols, 1), block(kBlock);
+    constexpr int P = kGeneralDepth;
+    if (!general) {
+        if (s.k == 3) pick_forward<T, 3, 1>(s, p, st);
+        else pick_forward<T, 4, 2>(s, p, st);
+    } else if (s.k == 3 && s.skip_type == 1) {
+        hipLaunchKernelGGL((forward_scan<T, 3, 1, kGeneral, 1, P>), grid, block, 0, st, p);
+    } else if (s.k == 3) {
+        hipLaunchKernelGGL((forward_scan<T, 3, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+    } else if (s.skip_type == 2) {
+        hipLaunchKernelGGL((forward_scan<T, 4, 2, kGeneral, 1, P>), grid, block, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((forward_scan<T, 4, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+    }
+}
+
+template <typename T>
+void launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
+    const bool general = s.activation_type != 0 || s.is_custom != 0 || s.skip_type == 0;
+    const dim3 grid = grid_for(p.ncols, 1), block(kBlock);
+    constexpr int P = kGeneralDepth;
+    if (!general) {
+        if (s.k == 3) pick_backward<T, 3, 1>(s, p, st);
+        else pick_backward<T, 4, 2>(s, p, st);
+    } else if (s.k == 3 && s.skip_type == 1) {
+        hipLaunchKernelGGL((backward_scan<T, 3, 1, kGeneral, 1, P>), grid, block, 0, st, p);
+    } else if (s.k == 3) {
+        hipLaunchKernelGGL((backward_scan<T, 3, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+    } else if (s.skip_type == 2) {
+        hipLaunchKernelGGL((backward_scan<T, 4, 2, kGeneral, 1, P>), grid, block, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((backward_scan<T, 4, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+    }
+}
+
+}  // namespace sru_amd

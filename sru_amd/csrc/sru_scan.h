@@ -1,15 +1,20 @@
-// Device-side building blocks of the SRU recurrence kernels for gfx950.
+// Device-side code of the SRU recurrence kernels for gfx950.
 //
-// Mapping: one lane owns one column (batch b, direction, hidden j), col = b*D' + dir*d + j,
-// exactly the column order of the (L, B, D') tensors, so a 64-lane wavefront reads
-// 64*k consecutive elements of U per step and 64 consecutive elements of every other
-// stream. The time loop is strictly serial per column (the gates see the previous state),
-// so memory latency is hidden by depth, not by width: every lane keeps a ring of P
-// future steps in registers; each iteration consumes the oldest slot and refills it
-// with the step P ahead, so about P steps of loads are in flight per lane at all times.
+// Mapping. One lane owns COLS (1 or 2) adjacent columns; a column is one (batch b,
+// direction, hidden j) triple, col = b*D' + dir*d + j, exactly the column order of the
+// (L, B, D') tensors. A 64-lane wavefront therefore reads 64*COLS*k consecutive
+// elements of U per step and 64*COLS consecutive elements of every other stream, each
+// lane with one vector instruction per stream (float: dwordx3 / dwordx4; 16-bit
+// elements with COLS = 2: the same dword-granular mix, which is why the 16-bit kernels
+// pair columns).
 //
-// Columns of the second direction walk time backwards. The loop variable is the walk
-// step s (uniform over the wavefront); the time index is s or L-1-s per lane.
+// Latency hiding. The time loop is strictly serial per column (both gates see the
+// previous state), so memory latency is hidden by depth, not by width: every lane keeps
+// a ring of P future steps in registers; each iteration consumes the oldest slot and
+// refills it with the step P ahead.
+//
+// Directions. Columns of the second direction walk time backwards. The loop variable
+// is the walk step s (uniform over the wavefront); the time index is s or L-1-s per lane.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -22,54 +27,94 @@ constexpr int kBlock = 64;  // one wavefront per workgroup: finest dispatch gran
 struct half_bits { uint16_t v; };  // IEEE binary16 storage
 struct bf16_bits { uint16_t v; };  // bfloat16 storage
 
-// ---------------------------------------------------------------- element conversion
-__device__ __forceinline__ float to_float(float v) { return v; }
-__device__ __forceinline__ float to_float(half_bits v) {
-    return (float)__builtin_bit_cast(_Float16, v.v);
+// ---------------------------------------------------------------- 16-bit conversion
+template <typename T> __device__ __forceinline__ float bits_to_float(uint32_t h);  // h < 65536
+template <> __device__ __forceinline__ float bits_to_float<half_bits>(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
-__device__ __forceinline__ float to_float(bf16_bits v) {
-    return __builtin_bit_cast(float, (uint32_t)v.v << 16);
+template <> __device__ __forceinline__ float bits_to_float<bf16_bits>(uint32_t h) {
+    return __builtin_bit_cast(float, h << 16);
+}
+template <typename T> __device__ __forceinline__ uint32_t float_to_bits(float v);  // round to nearest even
+template <> __device__ __forceinline__ uint32_t float_to_bits<half_bits>(float v) {
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+template <> __device__ __forceinline__ uint32_t float_to_bits<bf16_bits>(float v) {
+    return __builtin_bit_cast(uint16_t, (__bf16)v);
+}
+// two floats -> one dword of two 16-bit elements (lo first), one packed conversion
+typedef float float2v __attribute__((ext_vector_type(2)));
+template <typename T> __device__ __forceinline__ uint32_t pack_pair(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack_pair<half_bits>(float lo, float hi) {
+    typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((float2v){lo, hi}, half2v));
+}
+template <> __device__ __forceinline__ uint32_t pack_pair<bf16_bits>(float lo, float hi) {
+    typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((float2v){lo, hi}, bf2v));
 }
 
-template <typename T> __device__ __forceinline__ T from_float(float v);
-template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
-template <> __device__ __forceinline__ half_bits from_float<half_bits>(float v) {
-    return half_bits{__builtin_bit_cast(uint16_t, (_Float16)v)};  // round to nearest even
-}
-template <> __device__ __forceinline__ bf16_bits from_float<bf16_bits>(float v) {
-    uint32_t u = __builtin_bit_cast(uint32_t, v);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_bits{(uint16_t)((u >> 16) | 0x40u)};  // NaN
-    u += 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-    return bf16_bits{(uint16_t)(u >> 16)};
+// ---------------------------------------------------------------- groups of N consecutive elements
+// A Group is what one lane moves per stream and step. It is loaded and stored whole so
+// that the compiler emits one vector instruction where alignment allows, and it stays
+// in its storage form inside the ring (16-bit pairs stay packed in dwords).
+constexpr int group_align(int bytes) {
+    return bytes % 16 == 0 ? 16 : bytes % 8 == 0 ? 8 : bytes % 4 == 0 ? 4 : 2;
 }
 
-// ---------------------------------------------------------------- packed groups of N elements
-// N consecutive elements moved by one instruction where the type allows it:
-// float x3 -> dwordx3, float x4 -> dwordx4, 16-bit x2 -> dword, 16-bit x4 -> dwordx2.
-template <typename T, int N> struct Pack;
-template <> struct alignas(4) Pack<float, 2> { float e[2]; };
-template <> struct alignas(4) Pack<float, 3> { float e[3]; };
-template <> struct alignas(16) Pack<float, 4> { float e[4]; };
-template <> struct alignas(4) Pack<half_bits, 2> { half_bits e[2]; };
-template <> struct alignas(2) Pack<half_bits, 3> { half_bits e[3]; };
-template <> struct alignas(8) Pack<half_bits, 4> { half_bits e[4]; };
-template <> struct alignas(4) Pack<bf16_bits, 2> { bf16_bits e[2]; };
-template <> struct alignas(2) Pack<bf16_bits, 3> { bf16_bits e[3]; };
-template <> struct alignas(8) Pack<bf16_bits, 4> { bf16_bits e[4]; };
+// storage kind: 0 float, 1 even count of 16-bit elements, 2 odd count of 16-bit elements
+template <typename T, int N> constexpr int group_kind() { return sizeof(T) == 4 ? 0 : (N % 2 == 0 ? 1 : 2); }
+
+template <typename T, int N, int KIND = group_kind<T, N>()> struct Group;
+
+template <int N>
+struct alignas(group_align(4 * N)) Group<float, N, 0> {
+    float e[N];
+    __device__ __forceinline__ float get(int i) const { return e[i]; }
+    __device__ __forceinline__ static Group make(const float (&v)[N]) {
+        Group g;
+#pragma unroll
+        for (int i = 0; i < N; ++i) g.e[i] = v[i];
+        return g;
+    }
+};
+
+// even count of 16-bit elements: dwords holding two each
+template <typename T, int N>
+struct alignas(group_align(2 * N)) Group<T, N, 1> {
+    uint32_t w[N / 2];
+    __device__ __forceinline__ float get(int i) const {
+        return bits_to_float<T>((i & 1) ? (w[i / 2] >> 16) : (w[i / 2] & 0xffffu));
+    }
+    __device__ __forceinline__ static Group make(const float (&v)[N]) {
+        Group g;
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i)
+            g.w[i] = pack_pair<T>(v[2 * i], v[2 * i + 1]);
+        return g;
+    }
+};
+
+// odd count of 16-bit elements (one column per lane): element-wise
+template <typename T, int N>
+struct alignas(2) Group<T, N, 2> {
+    uint16_t h[N];
+    __device__ __forceinline__ float get(int i) const { return bits_to_float<T>(h[i]); }
+    __device__ __forceinline__ static Group make(const float (&v)[N]) {
+        Group g;
+#pragma unroll
+        for (int i = 0; i < N; ++i) g.h[i] = (uint16_t)float_to_bits<T>(v[i]);
+        return g;
+    }
+};
 
 template <typename T, int N>
-__device__ __forceinline__ void load_group(const T *p, float (&out)[N]) {
-    const Pack<T, N> v = *reinterpret_cast<const Pack<T, N> *>(p);
-#pragma unroll
-    for (int i = 0; i < N; ++i) out[i] = to_float(v.e[i]);
+__device__ __forceinline__ Group<T, N> load_group(const T *p) {
+    return *reinterpret_cast<const Group<T, N> *>(p);
 }
-
 template <typename T, int N>
-__device__ __forceinline__ void store_group(T *p, const float (&in)[N]) {
-    Pack<T, N> v;
-#pragma unroll
-    for (int i = 0; i < N; ++i) v.e[i] = from_float<T>(in[i]);
-    *reinterpret_cast<Pack<T, N> *>(p) = v;
+__device__ __forceinline__ void store_group(T *p, const float (&v)[N]) {
+    *reinterpret_cast<Group<T, N> *>(p) = Group<T, N>::make(v);
 }
 
 // ---------------------------------------------------------------- gate arithmetic
@@ -107,23 +152,23 @@ struct BwdParams {
     int32_t act, custom;
 };
 
-// ================================================================= forward scan
-// T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
-// U[..., 3]. MODE: see below. P: ring depth.
-//
-// The loop body must stay one straight line of code for the compiler to count the
-// outstanding loads exactly (a uniform branch inside it makes the inserted waits drain
-// the whole ring once per round). The fast kernels therefore take "is there a padding
-// mask" and "is the per-step state kept" as template bits; the general kernels read
-// those and the rarely used tanh / per-step weight_c options from the parameters.
-constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
+// The loop body must stay one straight line of code for the compiler to keep the ring
+// in fixed registers and count outstanding loads (a uniform branch inside it makes the
+// inserted waits drain the ring at every step). The fast kernels therefore take "is
+// there a padding mask" and "is the per-step state kept" as template bits; the general
+// kernels read those and the rarely used tanh / per-step weight_c options from the
+// parameter block.
 constexpr int kHasPad = 1;   // MODE bit (fast kernels): mask_pad given
 constexpr int kKeepC = 2;    // MODE bit (fast forward kernels): c is stored
+constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
 
-template <typename T, int K, int SKIP, int MODE, int P>
+// ================================================================= forward scan
+// T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
+// U[..., 3]. COLS: columns per lane (2 needs an even d). P: ring depth.
+template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
-    const int64_t col = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;  // lane's first column
     if (col >= p.ncols) return;
 
     const int Dp = p.Dp;
@@ -132,16 +177,20 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     const bool flip = j >= p.d;  // second direction; never true when dirs == 1 (d == D')
     const bool custom = GENERAL && p.custom;
     const bool use_tanh = GENERAL && p.act;
+    const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
+    const bool keep_c = GENERAL ? (p.c != nullptr) : ((MODE & kKeepC) != 0);
 
-    float wc1 = 0.f, wc2 = 0.f;
-    if (!custom) {
-        wc1 = static_cast<const float *>(p.wc)[j];
-        wc2 = static_cast<const float *>(p.wc)[Dp + j];
+    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], cur[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        wc1[c] = custom ? 0.f : static_cast<const float *>(p.wc)[j + c];
+        wc2[c] = custom ? 0.f : static_cast<const float *>(p.wc)[Dp + j + c];
+        b1[c] = p.bias[j + c];
+        b2[c] = p.bias[Dp + j + c];
+        m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
+        cur[c] = p.c0[col + c];
     }
-    const float b1 = p.bias[j], b2 = p.bias[Dp + j];
-    const float m = p.mask_c ? p.mask_c[col] : 1.0f;
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
-    float cur = p.c0[col];
 
     const int64_t L = p.L;
     const int64_t e0 = (flip ? (L - 1) : 0) * p.ncols + col;  // element of the first walk step
@@ -149,30 +198,28 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     const T *up = static_cast<const T *>(p.u) + e0 * K;
     const T *xp = (SKIP == 1) ? static_cast<const T *>(p.x) + e0 : nullptr;
     const T *vp = custom ? static_cast<const T *>(p.wc) + e0 * 2 : nullptr;
-    const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
-    const bool keep_c = GENERAL ? (p.c != nullptr) : ((MODE & kKeepC) != 0);
     const uint8_t *pp = has_pad ? p.pad + (flip ? (L - 1) : 0) * p.B + b : nullptr;
     const int64_t ps = flip ? -p.B : p.B;
     T *hp = static_cast<T *>(p.h) + e0;
     T *cp = keep_c ? static_cast<T *>(p.c) + e0 : nullptr;
 
     struct Slot {
-        float u[K];
-        float x;
-        float w[2];
+        Group<T, COLS * K> u;
+        Group<T, COLS> x;
+        Group<T, COLS * 2> w;
         uint32_t pad;
     };
     Slot ring[P];
 
     auto fetch = [&](Slot &s) {
-        load_group<T, K>(up, s.u);
+        s.u = load_group<T, COLS * K>(up);
         up += es * K;
         if (SKIP == 1) {
-            s.x = to_float(*xp);
+            s.x = load_group<T, COLS>(xp);
             xp += es;
         }
         if (custom) {
-            load_group<T, 2>(vp, s.w);
+            s.w = load_group<T, COLS * 2>(vp);
             vp += es * 2;
         }
         s.pad = 0;
@@ -183,25 +230,32 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     };
 
     auto consume = [&](const Slot &s) {
-        const float w1 = custom ? s.w[0] : wc1;
-        const float w2 = custom ? s.w[1] : wc2;
-        const float g1 = sigmoid(s.u[1] + w1 * cur + b1);
-        const float g2 = sigmoid(s.u[2] + w2 * cur + b2);
-        const float cn = (cur - s.u[0]) * g1 + s.u[0];
-        const float val = use_tanh ? tanhf(cn) : cn;
-        float hv;
-        if (SKIP != 0) {
-            const float xv = (SKIP == 1) ? s.x * sx : s.u[K - 1];
-            hv = (val - xv) * m * g2 + xv;
-        } else {
-            hv = val * m * g2;
-        }
         const bool padded = s.pad != 0;
-        cur = padded ? cur : cn;  // a padded step keeps the state ...
-        *hp = from_float<T>(padded ? 0.0f : hv);  // ... and emits zero
+        float hv[COLS], cv[COLS];
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            const float u0 = s.u.get(c * K), u1 = s.u.get(c * K + 1), u2 = s.u.get(c * K + 2);
+            const float w1 = custom ? s.w.get(2 * c) : wc1[c];
+            const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
+            const float g1 = sigmoid(u1 + w1 * cur[c] + b1[c]);
+            const float g2 = sigmoid(u2 + w2 * cur[c] + b2[c]);
+            const float cn = (cur[c] - u0) * g1 + u0;
+            const float val = use_tanh ? tanhf(cn) : cn;
+            float out;
+            if (SKIP != 0) {
+                const float xv = (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
+                out = (val - xv) * m[c] * g2 + xv;
+            } else {
+                out = val * m[c] * g2;
+            }
+            cur[c] = padded ? cur[c] : cn;   // a padded step keeps the state ...
+            hv[c] = padded ? 0.0f : out;     // ... and emits zero
+            cv[c] = cur[c];
+        }
+        store_group<T, COLS>(hp, hv);
         hp += es;
         if (keep_c) {
-            *cp = from_float<T>(cur);
+            store_group<T, COLS>(cp, cv);
             cp += es;
         }
     };
@@ -231,18 +285,19 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             }
         }
     }
-    p.c_last[col] = cur;
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
 }
 
 // ================================================================= backward scan
 // Walks each column's steps in reverse order, carrying d(loss)/d(state). The gates are
 // recomputed from U and the stored previous state. Sums of the weight_c and bias
-// gradients over time stay in four registers per lane and leave the kernel as
-// per-column partials; reduce_partials() then adds them over the batch in a fixed order.
-template <typename T, int K, int SKIP, int MODE, int P>
+// gradients over time stay in registers and leave the kernel as per-column partials;
+// reduce_partials() then adds them over the batch in a fixed order.
+template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
-    const int64_t col = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
 
     const int Dp = p.Dp;
@@ -251,16 +306,23 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     const bool flip = j >= p.d;
     const bool custom = GENERAL && p.custom;
     const bool use_tanh = GENERAL && p.act;
+    const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
 
-    float wc1 = 0.f, wc2 = 0.f;
-    if (!custom) {
-        wc1 = static_cast<const float *>(p.wc)[j];
-        wc2 = static_cast<const float *>(p.wc)[Dp + j];
+    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
+    float cur[COLS];  // d loss / d state
+    float gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        wc1[c] = custom ? 0.f : static_cast<const float *>(p.wc)[j + c];
+        wc2[c] = custom ? 0.f : static_cast<const float *>(p.wc)[Dp + j + c];
+        b1[c] = p.bias[j + c];
+        b2[c] = p.bias[Dp + j + c];
+        m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
+        c_init[c] = p.c0[col + c];
+        cur[c] = p.glast[col + c];
+        gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
     }
-    const float b1 = p.bias[j], b2 = p.bias[Dp + j];
-    const float m = p.mask_c ? p.mask_c[col] : 1.0f;
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
-    const float c_init = p.c0[col];
 
     const int64_t L = p.L;
     // The backward walk starts where the forward walk ended.
@@ -272,43 +334,45 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     const T *vp = custom ? static_cast<const T *>(p.wc) + e0 * 2 : nullptr;
     const T *ghp = static_cast<const T *>(p.gh) + e0;
     const T *cpp = static_cast<const T *>(p.c) + e0 + es;  // state before the step
-    const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
     const uint8_t *pp = has_pad ? p.pad + t_start * p.B + b : nullptr;
     const int64_t ps = flip ? p.B : -p.B;
     T *gup = static_cast<T *>(p.gu) + e0 * K;
     T *gxp = (SKIP == 1) ? static_cast<T *>(p.gx) + e0 : nullptr;
     T *gvp = custom ? static_cast<T *>(p.gwc_steps) + e0 * 2 : nullptr;
 
-    float cur = p.glast[col];                                       // d loss / d state
-    float cv = to_float(static_cast<const T *>(p.c)[e0]);           // state after the step
-    float gw1 = 0.f, gw2 = 0.f, gb1 = 0.f, gb2 = 0.f;
+    float cv[COLS];  // state after the step being visited
+    {
+        const Group<T, COLS> g = load_group<T, COLS>(static_cast<const T *>(p.c) + e0);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) cv[c] = g.get(c);
+    }
 
     struct Slot {
-        float u[K];
-        float x;
-        float w[2];
-        float gh;
-        float cprev;
+        Group<T, COLS * K> u;
+        Group<T, COLS> x;
+        Group<T, COLS * 2> w;
+        Group<T, COLS> gh;
+        Group<T, COLS> cprev;  // state before the step, as stored by the forward pass
+        bool first;            // the column's first forward step: the state before it is c_init
         uint32_t pad;
     };
     Slot ring[P];
 
-    // `last` = this is the column's first forward step: its previous state is c_init.
-    auto fetch = [&](Slot &s, bool last) {
-        load_group<T, K>(up, s.u);
+    auto fetch = [&](Slot &s, bool first) {
+        s.u = load_group<T, COLS * K>(up);
         up += es * K;
         if (SKIP == 1) {
-            s.x = to_float(*xp);
+            s.x = load_group<T, COLS>(xp);
             xp += es;
         }
         if (custom) {
-            load_group<T, 2>(vp, s.w);
+            s.w = load_group<T, COLS * 2>(vp);
             vp += es * 2;
         }
-        s.gh = to_float(*ghp);
+        s.gh = load_group<T, COLS>(ghp);
         ghp += es;
-        s.cprev = c_init;
-        if (!last) s.cprev = to_float(*cpp);
+        s.first = first;
+        if (!first) s.cprev = load_group<T, COLS>(cpp);
         cpp += es;
         s.pad = 0;
         if (has_pad) {
@@ -318,46 +382,51 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     };
 
     auto consume = [&](const Slot &s) {
-        const float w1 = custom ? s.w[0] : wc1;
-        const float w2 = custom ? s.w[1] : wc2;
-        const float cp = s.cprev;
-        const float u0 = s.u[0];
-        const float g1 = sigmoid(s.u[1] + w1 * cp + b1);
-        const float g2 = sigmoid(s.u[2] + w2 * cp + b2);
-        const float val = use_tanh ? tanhf(cv) : cv;
-        const float dact = use_tanh ? (1.0f - val * val) : 1.0f;
-        const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? s.x * sx : s.u[K - 1];
-        const float gh = s.gh;
         const bool padded = s.pad != 0;
+        float gu[COLS * K], gx[COLS], gv[COLS * 2];
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            const float w1 = custom ? s.w.get(2 * c) : wc1[c];
+            const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
+            const float cp = s.first ? c_init[c] : s.cprev.get(c);
+            const float u0 = s.u.get(c * K);
+            const float g1 = sigmoid(s.u.get(c * K + 1) + w1 * cp + b1[c]);
+            const float g2 = sigmoid(s.u.get(c * K + 2) + w2 * cp + b2[c]);
+            const float val = use_tanh ? tanhf(cv[c]) : cv[c];
+            const float dact = use_tanh ? (1.0f - val * val) : 1.0f;
+            const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
+            const float gh = s.gh.get(c);
 
-        const float gg2 = gh * (val - xv) * m * (g2 * (1.0f - g2));
-        const float gc = gh * m * (g2 * dact) + cur;
-        const float gg1 = gc * (cp - u0) * (g1 * (1.0f - g1));
-        const float gskip = gh * (1.0f - g2 * m);
-        const float ncur = gc * g1 + gg1 * w1 + gg2 * w2;
+            const float gg2 = gh * (val - xv) * m[c] * (g2 * (1.0f - g2));
+            const float gc = gh * m[c] * (g2 * dact) + cur[c];
+            const float gg1 = gc * (cp - u0) * (g1 * (1.0f - g1));
+            const float gskip = gh * (1.0f - g2 * m[c]);
+            const float ncur = gc * g1 + gg1 * w1 + gg2 * w2;
 
-        float gu[K];
-        gu[0] = padded ? 0.0f : gc * (1.0f - g1);
-        gu[1] = padded ? 0.0f : gg1;
-        gu[2] = padded ? 0.0f : gg2;
-        if (K == 4) gu[K - 1] = (padded || SKIP != 2) ? 0.0f : gskip;
-        store_group<T, K>(gup, gu);
+            gu[c * K] = padded ? 0.0f : gc * (1.0f - g1);
+            gu[c * K + 1] = padded ? 0.0f : gg1;
+            gu[c * K + 2] = padded ? 0.0f : gg2;
+            if (K == 4) gu[c * K + K - 1] = (padded || SKIP != 2) ? 0.0f : gskip;
+            gx[c] = padded ? 0.0f : gskip * sx;
+            gv[2 * c] = padded ? 0.0f : gg1 * cp;
+            gv[2 * c + 1] = padded ? 0.0f : gg2 * cp;
+            gb1[c] += padded ? 0.0f : gg1;
+            gw1[c] += padded ? 0.0f : gg1 * cp;
+            gb2[c] += padded ? 0.0f : gg2;
+            gw2[c] += padded ? 0.0f : gg2 * cp;
+            cur[c] = padded ? cur[c] : ncur;
+            cv[c] = cp;  // the state before this step is the state after the next one visited
+        }
+        store_group<T, COLS * K>(gup, gu);
         gup += es * K;
         if (SKIP == 1) {
-            *gxp = from_float<T>(padded ? 0.0f : gskip * sx);
+            store_group<T, COLS>(gxp, gx);
             gxp += es;
         }
         if (custom) {
-            const float gv[2] = {padded ? 0.0f : gg1 * cp, padded ? 0.0f : gg2 * cp};
-            store_group<T, 2>(gvp, gv);
+            store_group<T, COLS * 2>(gvp, gv);
             gvp += es * 2;
         }
-        gb1 += padded ? 0.0f : gg1;
-        gw1 += padded ? 0.0f : gg1 * cp;
-        gb2 += padded ? 0.0f : gg2;
-        gw2 += padded ? 0.0f : gg2 * cp;
-        cur = padded ? cur : ncur;
-        cv = cp;  // the state before this step is the state after the next one visited
     };
 
 #pragma unroll
@@ -384,49 +453,13 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
         }
     }
 
-    p.ginit[col] = cur;
-    p.partial[col] = gw1;
-    p.partial[p.ncols + col] = gw2;
-    p.partial[2 * p.ncols + col] = gb1;
-    p.partial[3 * p.ncols + col] = gb2;
-}
-
-// ================================================================= batch reduction
-// partial (4, B, D') -> grad_wc (2, D'), grad_bias (2, D'). One workgroup per 64 hidden
-// indices and per quantity; its 16 wavefronts take every 16th batch row each (loads of
-// a wavefront are 256 contiguous bytes), accumulate in double and are combined through
-// LDS in a fixed order, so the result does not depend on scheduling.
-constexpr int kReduceSlices = 16;
-
-__global__ void __launch_bounds__(64 * kReduceSlices)
-reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t B, int32_t Dp) {
-    __shared__ double acc[kReduceSlices][64];
-    const int lane = threadIdx.x & 63;
-    const int slice = threadIdx.x >> 6;
-    const int j = blockIdx.x * 64 + lane;
-    const int q = blockIdx.y;  // 0 gwc1, 1 gwc2, 2 gbias1, 3 gbias2
-    double sum = 0.0;
-    if (j < Dp) {
-        const float *src = partial + ((int64_t)q * B) * Dp + j;
-        int64_t b = slice;
-        for (; b + 3 * kReduceSlices < B; b += 4 * kReduceSlices) {  // 4 loads in flight
-            const float v0 = src[b * Dp], v1 = src[(b + kReduceSlices) * Dp];
-            const float v2 = src[(b + 2 * kReduceSlices) * Dp], v3 = src[(b + 3 * kReduceSlices) * Dp];
-            sum += (double)v0;
-            sum += (double)v1;
-            sum += (double)v2;
-            sum += (double)v3;
-        }
-        for (; b < B; b += kReduceSlices) sum += (double)src[b * Dp];
-    }
-    acc[slice][lane] = sum;
-    __syncthreads();
-    if (slice == 0 && j < Dp) {
-        double total = acc[0][lane];
 #pragma unroll
-        for (int s = 1; s < kReduceSlices; ++s) total += acc[s][lane];
-        float *dst = (q < 2) ? grad_wc : grad_bias;
-        if (dst) dst[(q & 1) * Dp + j] = (float)total;
+    for (int c = 0; c < COLS; ++c) {
+        p.ginit[col + c] = cur[c];
+        p.partial[col + c] = gw1[c];
+        p.partial[p.ncols + col + c] = gw2[c];
+        p.partial[2 * p.ncols + col + c] = gb1[c];
+        p.partial[3 * p.ncols + col + c] = gb2[c];
     }
 }
 
