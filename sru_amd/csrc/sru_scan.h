@@ -108,13 +108,51 @@ struct alignas(2) Group<T, N, 2> {
     }
 };
 
-template <typename T, int N>
+// NT: mark the access non-temporal (streamed once; do not keep the line in the caches).
+// A group travels as 1, 2, 3 or 4 dwords; odd 16-bit groups stay ordinary accesses.
+template <int WORDS> struct Words {
+    typedef uint32_t type __attribute__((ext_vector_type(WORDS), aligned(4)));
+};
+template <> struct Words<1> { typedef uint32_t type; };
+
+template <typename T, int N, bool NT = false>
 __device__ __forceinline__ Group<T, N> load_group(const T *p) {
-    return *reinterpret_cast<const Group<T, N> *>(p);
+    typedef Group<T, N> G;
+    if constexpr (NT && sizeof(G) % 4 == 0 && sizeof(G) <= 16) {
+        constexpr int W = sizeof(G) / 4;
+        typedef typename Words<W>::type vec_t;
+        const vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p));
+        uint32_t w[W];
+        if constexpr (W == 1) {
+            w[0] = v;
+        } else {
+#pragma unroll
+            for (int i = 0; i < W; ++i) w[i] = v[i];
+        }
+        return __builtin_bit_cast(G, w);
+    } else {
+        return *reinterpret_cast<const G *>(p);
+    }
 }
-template <typename T, int N>
+template <typename T, int N, bool NT = false>
 __device__ __forceinline__ void store_group(T *p, const float (&v)[N]) {
-    *reinterpret_cast<Group<T, N> *>(p) = Group<T, N>::make(v);
+    typedef Group<T, N> G;
+    if constexpr (NT && sizeof(G) % 4 == 0 && sizeof(G) <= 16) {
+        constexpr int W = sizeof(G) / 4;
+        typedef typename Words<W>::type vec_t;
+        struct Raw { uint32_t w[W]; };
+        const Raw r = __builtin_bit_cast(Raw, G::make(v));
+        vec_t out;
+        if constexpr (W == 1) {
+            out = r.w[0];
+        } else {
+#pragma unroll
+            for (int i = 0; i < W; ++i) out[i] = r.w[i];
+        }
+        __builtin_nontemporal_store(out, reinterpret_cast<vec_t *>(p));
+    } else {
+        *reinterpret_cast<G *>(p) = G::make(v);
+    }
 }
 
 // ---------------------------------------------------------------- gate arithmetic
@@ -161,6 +199,8 @@ struct BwdParams {
 constexpr int kHasPad = 1;   // MODE bit (fast kernels): mask_pad given
 constexpr int kKeepC = 2;    // MODE bit (fast forward kernels): c is stored
 constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
+constexpr int kNtLoad = 8;   // MODE bit: stream loads are non-temporal
+constexpr int kNtStore = 16; // MODE bit: stream stores are non-temporal
 
 // ================================================================= forward scan
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
@@ -168,6 +208,7 @@ constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
 template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
+    constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;  // lane's first column
     if (col >= p.ncols) return;
 
@@ -212,14 +253,14 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     Slot ring[P];
 
     auto fetch = [&](Slot &s) {
-        s.u = load_group<T, COLS * K>(up);
+        s.u = load_group<T, COLS * K, NTL>(up);
         up += es * K;
         if (SKIP == 1) {
-            s.x = load_group<T, COLS>(xp);
+            s.x = load_group<T, COLS, NTL>(xp);
             xp += es;
         }
         if (custom) {
-            s.w = load_group<T, COLS * 2>(vp);
+            s.w = load_group<T, COLS * 2, NTL>(vp);
             vp += es * 2;
         }
         s.pad = 0;
@@ -252,10 +293,10 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             hv[c] = padded ? 0.0f : out;     // ... and emits zero
             cv[c] = cur[c];
         }
-        store_group<T, COLS>(hp, hv);
+        store_group<T, COLS, NTS>(hp, hv);
         hp += es;
         if (keep_c) {
-            store_group<T, COLS>(cp, cv);
+            store_group<T, COLS, NTS>(cp, cv);
             cp += es;
         }
     };
@@ -297,6 +338,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
 template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
+    constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
 
@@ -359,20 +401,20 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     Slot ring[P];
 
     auto fetch = [&](Slot &s, bool first) {
-        s.u = load_group<T, COLS * K>(up);
+        s.u = load_group<T, COLS * K, NTL>(up);
         up += es * K;
         if (SKIP == 1) {
-            s.x = load_group<T, COLS>(xp);
+            s.x = load_group<T, COLS, NTL>(xp);
             xp += es;
         }
         if (custom) {
-            s.w = load_group<T, COLS * 2>(vp);
+            s.w = load_group<T, COLS * 2, NTL>(vp);
             vp += es * 2;
         }
-        s.gh = load_group<T, COLS>(ghp);
+        s.gh = load_group<T, COLS, NTL>(ghp);
         ghp += es;
         s.first = first;
-        if (!first) s.cprev = load_group<T, COLS>(cpp);
+        if (!first) s.cprev = load_group<T, COLS, NTL>(cpp);
         cpp += es;
         s.pad = 0;
         if (has_pad) {
@@ -417,14 +459,14 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
             cur[c] = padded ? cur[c] : ncur;
             cv[c] = cp;  // the state before this step is the state after the next one visited
         }
-        store_group<T, COLS * K>(gup, gu);
+        store_group<T, COLS * K, NTS>(gup, gu);
         gup += es * K;
         if (SKIP == 1) {
-            store_group<T, COLS>(gxp, gx);
+            store_group<T, COLS, NTS>(gxp, gx);
             gxp += es;
         }
         if (custom) {
-            store_group<T, COLS * 2>(gvp, gv);
+            store_group<T, COLS * 2, NTS>(gvp, gv);
             gvp += es * 2;
         }
     };
