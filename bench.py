@@ -77,6 +77,10 @@ def main():
     ap.add_argument("--dtype", default="f32", choices=sorted(DT_BYTES))
     ap.add_argument("--sets", type=int, default=4, help="rotating buffer sets")
     ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
+    ap.add_argument("--full-state", action="store_true",
+                    help="keep the state after every step between forward and backward, as the "
+                         "reference does, instead of float checkpoints every 8 steps (the path "
+                         "the autograd Function of this package takes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "
@@ -98,7 +102,10 @@ def main():
     tdt = TORCH_DT[args.dtype]
     es = DT_BYTES[args.dtype]
     lib = _lib.load()
-    shape = _lib.Shape(L, B, d, dirs, k, 0, 1 if k == 3 else 2, 0, CODE[args.dtype])
+    ckpt = not args.full_state and not fwd_only
+    shape = _lib.Shape(L, B, d, dirs, k, 0, 1 if k == 3 else 2, 0, CODE[args.dtype],
+                       _lib.STATE_INTERVAL if ckpt else 1)
+    state_rows = lib.sru_amd_state_bytes(ctypes.byref(shape)) // (B * Dp * (4 if ckpt else DT_BYTES[args.dtype]))
 
     g = torch.Generator(device=dev).manual_seed(1234)
     sets = []
@@ -108,7 +115,7 @@ def main():
             x=torch.randn(L, B, Dp, device=dev, generator=g).to(tdt),
             gh=torch.randn(L, B, Dp, device=dev, generator=g).to(tdt),
             h=torch.empty(L, B, Dp, device=dev, dtype=tdt),
-            c=torch.empty(L, B, Dp, device=dev, dtype=tdt),
+            c=torch.empty(state_rows, B, Dp, device=dev, dtype=torch.float32 if ckpt else tdt),
             gu=torch.empty(L, B, Dp * k, device=dev, dtype=tdt),
             gx=torch.empty(L, B, Dp, device=dev, dtype=tdt),
         )
@@ -188,7 +195,7 @@ def main():
     bwd_us = 1e3 * sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
     traffic = None   # HBM bytes per backward launch from the committed rocprofv3 counter runs
     tfile = os.path.join(ROOT, "profiles", "traffic_bi_d1024_L256_B64_%s.json" % args.dtype)
-    if args.workload == "headline" and os.path.exists(tfile):
+    if args.workload == "headline" and ckpt and os.path.exists(tfile):
         traffic = json.load(open(tfile))["backward_scan"]["traffic_bytes"]
     fwd_bytes = (5 if fwd_only else 6) * es * cells   # reads U (k) and x (k=3), writes h and (training) c
     bwd_bytes = 10 * es * cells    # reads U (k), x (k=3), c, grad_h; writes grad_u (k), grad_x (k=3)
@@ -204,8 +211,9 @@ def main():
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": name, "length": L, "batch": B, "hidden_per_direction": d,
                    "directions": dirs, "k": k, "pass": "forward+backward, one layer",
+                   "state_between_passes": "float checkpoints every 8 steps" if ckpt else "every step",
                    "buffer_sets": args.sets},
-        "roofline": {"bound": "hbm", "kernel": "backward_scan (+ reduce_partials)",
+        "roofline": {"bound": "hbm", "kernel": ("backward_scan_ckpt" if ckpt else "backward_scan") + " (+ reduce_partials)",
                      "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_us": bwd_us},

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define SRU_AMD_ABI_VERSION 1
+#define SRU_AMD_ABI_VERSION 2
 
 enum sru_amd_dtype {
     SRU_AMD_F32 = 0,
@@ -76,7 +76,17 @@ typedef struct sru_amd_shape {
     int32_t skip_type;       /* 0 none; 1 from x (k == 3); 2 from U[..., 3] (k == 4) */
     int32_t is_custom;       /* 0: weight_c (2, D'); 1: per step (L, B, D', 2) */
     int32_t dtype;           /* enum sru_amd_dtype */
+    int32_t state_interval;  /* what `c` holds between forward and backward:
+                              * 0 or 1: the state after every step, (L, B, D') in `dtype`, as
+                              *   the reference keeps it (sru_cuda_kernel.cu:72,:436);
+                              * SRU_AMD_STATE_INTERVAL: float checkpoints only, one row per
+                              *   SRU_AMD_STATE_INTERVAL steps of each column's walk,
+                              *   (max(1, L / SRU_AMD_STATE_INTERVAL), B, D') float; the backward
+                              *   call rebuilds the states in between. Needs activation_type 0,
+                              *   is_custom 0 and a skip term. No counterpart in the reference. */
 } sru_amd_shape;
+
+#define SRU_AMD_STATE_INTERVAL 8
 
 /* Forward scan. Replaces sru_cuda::sru_forward_simple, sru_bi_forward_simple,
  * sru_forward and sru_bi_forward (sru/csrc/sru_cuda_impl.cpp:177-207,:255-285,
@@ -85,8 +95,8 @@ typedef struct sru_amd_shape {
  *   x        required iff skip_type == 1
  *   mask_c   NULL = no dropout mask
  *   mask_pad NULL = no padding
- *   c        per-step state kept for the backward pass; NULL = do not store it
- *            (inference)
+ *   c        state kept for the backward pass, sru_amd_state_bytes() bytes laid out as
+ *            shape->state_interval says; NULL = do not store it (inference)
  *   c_last   state after the last step of each column's walk: what the
  *            reference assembles as cat(c[-1, :, :d], c[0, :, d:]) */
 int sru_amd_forward(const sru_amd_shape *shape,
@@ -94,6 +104,10 @@ int sru_amd_forward(const sru_amd_shape *shape,
                     const float *bias, const float *c_init, const float *mask_c,
                     const uint8_t *mask_pad, const float *scale_x,
                     void *h, void *c, float *c_last, void *stream);
+
+/* Bytes of the state buffer `c` that sru_amd_forward fills and sru_amd_backward reads for
+ * `shape`, according to shape->state_interval (0 on a bad shape). */
+size_t sru_amd_state_bytes(const sru_amd_shape *shape);
 
 /* Bytes of device scratch sru_amd_backward needs for `shape` (0 on a bad
  * shape). The scratch holds per-column partial sums of the weight_c and bias
@@ -105,7 +119,7 @@ size_t sru_amd_backward_workspace_bytes(const sru_amd_shape *shape);
  * :415-518) together with what sru/cuda_functional.py:204-207 and :253-260 run
  * around them: the x * scale_x pass, grad_x *= scale_x and the batch sums of
  * the weight_c / bias gradients.
- *   c         the per-step state the forward call stored
+ *   c         the state buffer the forward call filled (same shape->state_interval)
  *   grad_x    required iff skip_type == 1; already multiplied by scale_x
  *   grad_wc   (2, D') float summed over time and batch, or, when is_custom,
  *             (L, B, D', 2) in `dtype`

@@ -10,7 +10,8 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # SRU_AMD_LIBRARY points at another build of the same library (tuning builds)
 LIB_PATH = os.environ.get("SRU_AMD_LIBRARY") or os.path.join(_HERE, "libsru_amd.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
+STATE_INTERVAL = 8   # SRU_AMD_STATE_INTERVAL
 
 F32, F16, BF16 = 0, 1, 2
 
@@ -27,6 +28,7 @@ class Shape(ctypes.Structure):
         ("skip_type", ctypes.c_int32),
         ("is_custom", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
+        ("state_interval", ctypes.c_int32),
     ]
 
 
@@ -34,6 +36,7 @@ _P = ctypes.c_void_p
 SIGNATURES = {
     # name: (restype, argtypes) exactly as declared in include/sru_amd.h
     "sru_amd_forward": (ctypes.c_int, [ctypes.POINTER(Shape)] + [_P] * 12),
+    "sru_amd_state_bytes": (ctypes.c_size_t, [ctypes.POINTER(Shape)]),
     "sru_amd_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(Shape)]),
     "sru_amd_backward": (ctypes.c_int, [ctypes.POINTER(Shape)] + [_P] * 17 + [ctypes.c_size_t, _P]),
     "sru_amd_status_string": (ctypes.c_char_p, [ctypes.c_int]),

@@ -12,6 +12,8 @@ namespace {
 
 using namespace sru_amd;
 
+static_assert(SRU_AMD_STATE_INTERVAL == kCkptInterval, "header and kernels disagree");
+
 size_t elem_size(int dtype) { return dtype == SRU_AMD_F32 ? 4 : 2; }
 
 bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -30,6 +32,12 @@ int check_shape(const sru_amd_shape *s) {
     if (s->is_custom != 0 && s->is_custom != 1) return SRU_AMD_ERR_BAD_FLAGS;
     if (s->dtype != SRU_AMD_F32 && s->dtype != SRU_AMD_F16 && s->dtype != SRU_AMD_BF16)
         return SRU_AMD_ERR_BAD_DTYPE;
+    if (s->state_interval != 0 && s->state_interval != 1 && s->state_interval != SRU_AMD_STATE_INTERVAL)
+        return SRU_AMD_ERR_BAD_FLAGS;
+    // checkpointed state exists only for the fast kernels
+    if (s->state_interval == SRU_AMD_STATE_INTERVAL &&
+        (s->activation_type != 0 || s->is_custom != 0 || s->skip_type == 0))
+        return SRU_AMD_ERR_BAD_FLAGS;
     // D' must fit an int, the grid must fit 2^31-1 workgroups and the largest stream
     // (L*B*D'*k elements) must stay far inside the 64-bit byte offsets the kernels use.
     const int64_t lim = INT64_C(1) << 31;
@@ -71,7 +79,8 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
     if (s.skip_type == 1 && !x) return SRU_AMD_ERR_NULL_POINTER;
     const size_t es = elem_size(s.dtype);
     const size_t group = (s.k == 4) ? 4 * es : es;  // a k=4 group moves as one vector
-    if (!aligned(u, group) || !aligned(h, es) || (c && !aligned(c, es)) ||
+    const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
+    if (!aligned(u, group) || !aligned(h, es) || (c && !aligned(c, ckpt ? 4 : es)) ||
         (s.skip_type == 1 && !aligned(x, es)) || !aligned(weight_c, s.is_custom ? 2 * es : 4) ||
         !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(c_last, 4) ||
         (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
@@ -79,7 +88,9 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
 
     FwdParams p{};
     p.u = u; p.x = x; p.wc = weight_c; p.bias = bias; p.c0 = c_init; p.mask_c = mask_c;
-    p.pad = mask_pad; p.scale_x = scale_x; p.h = h; p.c = c; p.c_last = c_last;
+    p.pad = mask_pad; p.scale_x = scale_x; p.h = h; p.c_last = c_last;
+    p.c = ckpt ? nullptr : c;
+    p.ckpt = ckpt ? static_cast<float *>(c) : nullptr;
     p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
     p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
 
@@ -89,6 +100,16 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
     else if (s.dtype == SRU_AMD_F16) launch_forward<half_bits>(s, p, st);
     else launch_forward<bf16_bits>(s, p, st);
     return hipGetLastError() == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+}
+
+size_t sru_amd_state_bytes(const sru_amd_shape *shape) {
+    if (check_shape(shape) != SRU_AMD_OK) return 0;
+    const size_t ncols = (size_t)(shape->batch * shape->hidden * shape->dirs);
+    if (shape->state_interval == SRU_AMD_STATE_INTERVAL) {
+        const size_t rows = (size_t)(shape->length / SRU_AMD_STATE_INTERVAL);
+        return (rows ? rows : 1) * ncols * sizeof(float);
+    }
+    return (size_t)shape->length * ncols * elem_size(shape->dtype);
 }
 
 size_t sru_amd_backward_workspace_bytes(const sru_amd_shape *shape) {
@@ -110,7 +131,8 @@ int sru_amd_backward(const sru_amd_shape *shape, const void *u, const void *x, c
     if (s.skip_type == 1 && (!x || !grad_x)) return SRU_AMD_ERR_NULL_POINTER;
     const size_t es = elem_size(s.dtype);
     const size_t group = (s.k == 4) ? 4 * es : es;
-    if (!aligned(u, group) || !aligned(grad_u, group) || !aligned(c, es) || !aligned(grad_h, es) ||
+    const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
+    if (!aligned(u, group) || !aligned(grad_u, group) || !aligned(c, ckpt ? 4 : es) || !aligned(grad_h, es) ||
         (s.skip_type == 1 && (!aligned(x, es) || !aligned(grad_x, es))) ||
         !aligned(weight_c, s.is_custom ? 2 * es : 4) || !aligned(grad_wc, s.is_custom ? 2 * es : 4) ||
         !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(grad_last, 4) || !aligned(grad_bias, 4) ||
@@ -122,7 +144,9 @@ int sru_amd_backward(const sru_amd_shape *shape, const void *u, const void *x, c
 
     BwdParams p{};
     p.u = u; p.x = x; p.wc = weight_c; p.bias = bias; p.c0 = c_init; p.mask_c = mask_c;
-    p.pad = mask_pad; p.scale_x = scale_x; p.c = c; p.gh = grad_h; p.glast = grad_last;
+    p.pad = mask_pad; p.scale_x = scale_x; p.gh = grad_h; p.glast = grad_last;
+    p.c = ckpt ? nullptr : c;
+    p.ckpt = ckpt ? static_cast<const float *>(c) : nullptr;
     p.gu = grad_u; p.gx = grad_x; p.gwc_steps = s.is_custom ? grad_wc : nullptr;
     p.ginit = grad_init; p.partial = static_cast<float *>(workspace);
     p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);

@@ -75,12 +75,16 @@ template <typename T, int K, int SKIP, int COLS>
 void fast_forward(const FwdParams &p, hipStream_t st) {
     constexpr int P = Tune<T>::kFwdDepth;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
-    const int mode = (p.pad ? kHasPad : 0) | (p.c ? kKeepC : 0);
+    // what is kept for the backward pass: nothing, the state after every step, or checkpoints
+    const int keep = p.ckpt ? kCkpt : (p.c ? kKeepC : 0);
+    const int mode = (p.pad ? kHasPad : 0) | keep;
     switch (mode) {
     case 0: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kFwdNt, COLS, P>), grid, block, 0, st, p); break;
     case kHasPad: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
     case kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kKeepC | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
-    default: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kKeepC | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
+    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kKeepC | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
+    case kCkpt: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kCkpt | kFwdNt, COLS, kCkptInterval>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kCkpt | kFwdNt, COLS, kCkptInterval>), grid, block, 0, st, p); break;
     }
 }
 
@@ -88,8 +92,14 @@ template <typename T, int K, int SKIP, int COLS>
 void fast_backward(const BwdParams &p, hipStream_t st) {
     constexpr int P = Tune<T>::kBwdDepth;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
-    if (p.pad) hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad | kBwdNt, COLS, P>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((backward_scan<T, K, SKIP, kBwdNt, COLS, P>), grid, block, 0, st, p);
+    if (p.ckpt) {
+        if (p.pad) hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt, COLS, kCkptInterval>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt, COLS, kCkptInterval>), grid, block, 0, st, p);
+    } else if (p.pad) {
+        hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad | kBwdNt, COLS, P>), grid, block, 0, st, p);
+    } else {
+        hipLaunchKernelGGL((backward_scan<T, K, SKIP, kBwdNt, COLS, P>), grid, block, 0, st, p);
+    }
 }
 
 template <typename T, int K, int SKIP>
@@ -103,7 +113,7 @@ void pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
 template <typename T, int K, int SKIP>
 void pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
     if constexpr (Tune<T>::kCols == 2) {
-        if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) return fast_backward<T, K, SKIP, 2>(p, st);
+        if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) return fast_backward<T, K, SKIP, 2>(p, st);  // p.c is null with checkpoints
     }
     fast_backward<T, K, SKIP, 1>(p, st);
 }

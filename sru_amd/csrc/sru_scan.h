@@ -170,6 +170,7 @@ struct FwdParams {
     const float *scale_x;
     void *h, *c;
     float *c_last;
+    float *ckpt;          // (L / kCkptInterval, B, D') float state checkpoints, or nullptr
     int64_t L, B, ncols;  // ncols = B * D'
     int32_t d, Dp;        // hidden per direction, D' = dirs * d
     int32_t act, custom;  // only read by the general kernels
@@ -181,6 +182,7 @@ struct BwdParams {
     const uint8_t *pad;
     const float *scale_x;
     const void *c, *gh;
+    const float *ckpt;    // state checkpoints written by the forward pass (checkpoint kernels)
     const float *glast;
     void *gu, *gx, *gwc_steps;  // gwc_steps: per-step weight_c gradient (custom only)
     float *ginit;
@@ -201,6 +203,15 @@ constexpr int kKeepC = 2;    // MODE bit (fast forward kernels): c is stored
 constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
 constexpr int kNtLoad = 8;   // MODE bit: stream loads are non-temporal
 constexpr int kNtStore = 16; // MODE bit: stream stores are non-temporal
+constexpr int kCkpt = 32;    // MODE bit (fast forward kernels): store a state checkpoint per chunk
+
+// Checkpointed state. Instead of the state after every step (4 bytes per cell written by
+// the forward pass and read again by the backward pass), the forward pass can keep only
+// the state after every kCkptInterval-th step of each column's walk, in float, whatever
+// the stream type: row r of the checkpoint array is the state after walk step
+// (r+1)*kCkptInterval - 1. The backward pass then rebuilds the states inside a chunk
+// from its checkpoint while it holds the chunk's U in registers anyway.
+constexpr int kCkptInterval = 8;
 
 // ================================================================= forward scan
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
@@ -209,6 +220,8 @@ template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
+    constexpr bool CKPT = (MODE & kCkpt) != 0;
+    static_assert(!CKPT || (P == kCkptInterval && !GENERAL), "a ring round is one checkpoint chunk");
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;  // lane's first column
     if (col >= p.ncols) return;
 
@@ -243,6 +256,12 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     const int64_t ps = flip ? -p.B : p.B;
     T *hp = static_cast<T *>(p.h) + e0;
     T *cp = keep_c ? static_cast<T *>(p.c) + e0 : nullptr;
+    float *kp = CKPT ? p.ckpt + col : nullptr;
+    auto checkpoint = [&]() {  // called after the last step of a chunk
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) kp[c] = cur[c];
+        kp += p.ncols;
+    };
 
     struct Slot {
         Group<T, COLS * K> u;
@@ -315,6 +334,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             // loads of a round at its end, where none of them has time to land.
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (CKPT) checkpoint();
     }
     for (; s0 < L; s0 += P) {  // last one or two rounds
 #pragma unroll
@@ -325,6 +345,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
                 consume(s);
             }
         }
+        if (CKPT && s0 + P <= L) checkpoint();
     }
 #pragma unroll
     for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
@@ -493,6 +514,177 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
                 consume(s);
             }
         }
+    }
+
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        p.ginit[col + c] = cur[c];
+        p.partial[col + c] = gw1[c];
+        p.partial[p.ncols + col + c] = gw2[c];
+        p.partial[2 * p.ncols + col + c] = gb1[c];
+        p.partial[3 * p.ncols + col + c] = gb2[c];
+    }
+}
+
+// ================================================================= backward scan from checkpoints
+// Same results as backward_scan, but the per-step state is rebuilt instead of read: the
+// walk is cut into chunks of TC steps, visited last to first. For a chunk the kernel
+// holds U, x and grad_h of its TC steps in registers, runs the forward recurrence from
+// the chunk's checkpoint (keeping both gates and the states), then the backward
+// recurrence over the same registers. Loads of the next chunk are issued before the
+// arithmetic of the current one. Per cell: reads U (k), x, grad_h and 4/TC bytes of
+// checkpoint; writes grad_u (k), grad_x.
+template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
+__global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) {
+    static_assert((MODE & kGeneral) == 0, "fast kernels only");
+    constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
+    constexpr bool HAS_PAD = (MODE & kHasPad) != 0;
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
+    if (col >= p.ncols) return;
+
+    const int Dp = p.Dp;
+    const int j = (int)(col % Dp);
+    const int64_t b = col / Dp;
+    const bool flip = j >= p.d;
+
+    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
+    float cur[COLS];  // d loss / d state
+    float gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        wc1[c] = static_cast<const float *>(p.wc)[j + c];
+        wc2[c] = static_cast<const float *>(p.wc)[Dp + j + c];
+        b1[c] = p.bias[j + c];
+        b2[c] = p.bias[Dp + j + c];
+        m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
+        c_init[c] = p.c0[col + c];
+        cur[c] = p.glast[col + c];
+        gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
+    }
+    const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
+
+    const int64_t L = p.L;
+    // forward-walk step s of this column sits at element ef + s * es
+    const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + col;
+    const int64_t es = flip ? -p.ncols : p.ncols;
+    const int64_t pf = (flip ? (L - 1) : 0) * p.B + b;
+    const int64_t ps = flip ? -p.B : p.B;
+    const T *ubase = static_cast<const T *>(p.u);
+    const T *xbase = static_cast<const T *>(p.x);
+    const T *ghbase = static_cast<const T *>(p.gh);
+    T *gubase = static_cast<T *>(p.gu);
+    T *gxbase = static_cast<T *>(p.gx);
+
+    struct Chunk {
+        Group<T, COLS * K> u[TC];
+        Group<T, COLS> x[TC];
+        Group<T, COLS> gh[TC];
+        uint32_t pad[TC];
+        float cstart[COLS];  // state before the chunk's first step
+    };
+
+    // n: number of valid steps in the chunk (TC except for a ragged last chunk)
+    auto load_chunk = [&](Chunk &k, int64_t ch, int n) {
+        const int64_t s0 = ch * TC;
+#pragma unroll
+        for (int i = 0; i < TC; ++i) {
+            if (i < n) {
+                const int64_t e = ef + (s0 + i) * es;
+                k.u[i] = load_group<T, COLS * K, NTL>(ubase + e * K);
+                if (SKIP == 1) k.x[i] = load_group<T, COLS, NTL>(xbase + e);
+                k.gh[i] = load_group<T, COLS, NTL>(ghbase + e);
+                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < COLS; ++c)
+            k.cstart[c] = (ch == 0) ? c_init[c] : p.ckpt[(ch - 1) * p.ncols + col + c];
+    };
+
+    auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) {
+        const int64_t s0 = ch * TC;
+        float st[TC + 1][COLS];  // st[i] = state before step i of the chunk
+        float g1[TC][COLS], g2[TC][COLS];
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) st[0][c] = k.cstart[c];
+#pragma unroll
+        for (int i = 0; i < TC; ++i) {
+            if (i < n) {
+                const bool padded = k.pad[i] != 0;
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) {
+                    const float cp = st[i][c];
+                    const float u0 = k.u[i].get(c * K);
+                    g1[i][c] = sigmoid(k.u[i].get(c * K + 1) + wc1[c] * cp + b1[c]);
+                    g2[i][c] = sigmoid(k.u[i].get(c * K + 2) + wc2[c] * cp + b2[c]);
+                    const float cn = (cp - u0) * g1[i][c] + u0;
+                    st[i + 1][c] = padded ? cp : cn;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = TC - 1; i >= 0; --i) {
+            if (i < n) {
+                const bool padded = k.pad[i] != 0;
+                float gu[COLS * K], gx[COLS];
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) {
+                    const float cp = st[i][c], val = st[i + 1][c];
+                    const float u0 = k.u[i].get(c * K);
+                    const float G1 = g1[i][c], G2 = g2[i][c];
+                    const float xv = (SKIP == 1) ? k.x[i].get(c) * sx : k.u[i].get(c * K + K - 1);
+                    const float gh = k.gh[i].get(c);
+
+                    const float gg2 = gh * (val - xv) * m[c] * (G2 * (1.0f - G2));
+                    const float gc = gh * m[c] * G2 + cur[c];
+                    const float gg1 = gc * (cp - u0) * (G1 * (1.0f - G1));
+                    const float gskip = gh * (1.0f - G2 * m[c]);
+                    const float ncur = gc * G1 + gg1 * wc1[c] + gg2 * wc2[c];
+
+                    gu[c * K] = padded ? 0.0f : gc * (1.0f - G1);
+                    gu[c * K + 1] = padded ? 0.0f : gg1;
+                    gu[c * K + 2] = padded ? 0.0f : gg2;
+                    if (K == 4) gu[c * K + K - 1] = padded ? 0.0f : gskip;
+                    gx[c] = padded ? 0.0f : gskip * sx;
+                    gb1[c] += padded ? 0.0f : gg1;
+                    gw1[c] += padded ? 0.0f : gg1 * cp;
+                    gb2[c] += padded ? 0.0f : gg2;
+                    gw2[c] += padded ? 0.0f : gg2 * cp;
+                    cur[c] = padded ? cur[c] : ncur;
+                }
+                const int64_t e = ef + (s0 + i) * es;
+                store_group<T, COLS * K, NTS>(gubase + e * K, gu);
+                if (SKIP == 1) store_group<T, COLS, NTS>(gxbase + e, gx);
+            }
+        }
+    };
+
+    const int64_t nfull = L / TC;
+    const int tail = (int)(L - nfull * TC);
+    Chunk ka, kb;
+    int64_t ch = nfull - 1;           // next full chunk to compute
+    if (ch >= 0) load_chunk(ka, ch, TC);
+    if (tail > 0) {                    // the ragged chunk is the last of the walk: visited first
+        load_chunk(kb, nfull, tail);
+        compute_chunk(kb, nfull, tail);
+    }
+    // Two chunks per iteration (ka, kb alternate) so that no register copies are needed and
+    // the loop body is a single block in which every prefetch is a real chunk.
+    while (ch >= 2) {
+        load_chunk(kb, ch - 1, TC);
+        compute_chunk(ka, ch, TC);
+        __builtin_amdgcn_sched_barrier(0);
+        load_chunk(ka, ch - 2, TC);
+        compute_chunk(kb, ch - 1, TC);
+        __builtin_amdgcn_sched_barrier(0);
+        ch -= 2;
+    }
+    if (ch == 1) {
+        load_chunk(kb, 0, TC);
+        compute_chunk(ka, 1, TC);
+        compute_chunk(kb, 0, TC);
+    } else if (ch == 0) {
+        compute_chunk(ka, 0, TC);
     }
 
 #pragma unroll

@@ -53,7 +53,8 @@ class _Problem:
     """Sizes and flags derived the way sru/cuda_functional.py:54-65 derives them."""
 
     def __init__(self, u: Tensor, x: Tensor, weight_c: Tensor, d_out: int,
-                 bidirectional: bool, has_skip_term: bool, activation_type: int):
+                 bidirectional: bool, has_skip_term: bool, activation_type: int,
+                 checkpoint_state: bool = False):
         if u.dtype not in _DTYPES:
             raise ValueError(f"U must be float32, float16 or bfloat16, not {u.dtype}")
         if not u.is_cuda:
@@ -74,9 +75,15 @@ class _Problem:
         self.activation_type = activation_type
         self.dtype = u.dtype
         self.squeeze = x.dim() == 2
+        # Between forward and backward keep float checkpoints of the state instead of the
+        # state after every step wherever the kernels support it (no tanh, no per-step
+        # weight_c, a skip term): the backward kernel rebuilds what lies in between.
+        self.checkpointed = bool(checkpoint_state and activation_type == 0
+                                 and not self.is_custom and self.skip_type != 0)
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
                                 activation_type, self.skip_type, self.is_custom,
-                                _DTYPES[u.dtype])
+                                _DTYPES[u.dtype],
+                                _lib.STATE_INTERVAL if self.checkpointed else 1)
 
     def group_bytes(self):
         es = 4 if self.dtype == torch.float32 else 2
@@ -120,10 +127,15 @@ def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, m
 
 def _run_forward(pb, u_, x_, wc_, bias_, init_, scale_, mask_c_, pad_, keep_c: bool):
     dev = u_.device
-    h = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
-    c = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev) if keep_c else None
-    c_last = torch.empty(pb.batch, pb.Dp, dtype=torch.float32, device=dev)
     lib = _lib.load()
+    h = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
+    c = None
+    if keep_c and pb.checkpointed:
+        rows = lib.sru_amd_state_bytes(ctypes.byref(pb.shape)) // (4 * pb.batch * pb.Dp)
+        c = torch.empty(rows, pb.batch, pb.Dp, dtype=torch.float32, device=dev)
+    elif keep_c:
+        c = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
+    c_last = torch.empty(pb.batch, pb.Dp, dtype=torch.float32, device=dev)
     with torch.cuda.device(dev):
         stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
         rc = lib.sru_amd_forward(ctypes.byref(pb.shape), _ptr(u_), _ptr(x_), _ptr(wc_), _ptr(bias_),
@@ -160,7 +172,8 @@ class ElementwiseRecurrence(Function):
     @staticmethod
     def forward(ctx, u, x, weight_c, bias, init, activation_type, d_out, bidirectional,
                 has_skip_term, scale_x, mask_c=None, mask_pad=None):
-        pb = _Problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type)
+        pb = _Problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type,
+                      checkpoint_state=True)
         prepared = _prepare_inputs(pb, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad)
         h, c, c_last = _run_forward(pb, *prepared, keep_c=True)
         ctx.problem = pb

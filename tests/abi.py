@@ -18,8 +18,10 @@ def p(t):
 class DeviceProblem:
     """Device copies of a Case in stream dtype `dt`; float32 for the small tensors."""
 
-    def __init__(self, case, dt="f32", device="cuda:0"):
-        self.case, self.dt = case, dt
+    def __init__(self, case, dt="f32", device="cuda:0", checkpointed=False):
+        """checkpointed: keep float state checkpoints between forward and backward
+        (shape.state_interval = SRU_AMD_STATE_INTERVAL) instead of the state after every step."""
+        self.case, self.dt, self.checkpointed = case, dt, checkpointed
         tdt = TORCH_DT[dt]
         dev = torch.device(device)
         big = lambda a: torch.tensor(a, dtype=tdt, device=dev).contiguous()
@@ -30,7 +32,8 @@ class DeviceProblem:
         self.bias, self.c0, self.gl, self.mask_c = small(c.bias), small(c.c0), small(c.gl), small(c.mask_c)
         self.scale = torch.tensor([c.scale], dtype=torch.float32, device=dev)
         self.pad = None if c.pad is None else torch.tensor(c.pad, dtype=torch.bool, device=dev).view(torch.uint8)
-        self.shape = _lib.Shape(c.L, c.B, c.d, c.dirs, c.k, c.act, c.skip_type, c.custom, CODE[dt])
+        self.shape = _lib.Shape(c.L, c.B, c.d, c.dirs, c.k, c.act, c.skip_type, c.custom, CODE[dt],
+                                _lib.STATE_INTERVAL if checkpointed else 1)
         self.dev, self.tdt = dev, tdt
 
     def rounded_case(self):
@@ -49,7 +52,11 @@ class DeviceProblem:
         mk = (lambda *s, dtype: torch.full(s, float("nan"), dtype=dtype, device=self.dev)) if poison else \
             (lambda *s, dtype: torch.empty(s, dtype=dtype, device=self.dev))
         self.h = mk(c.L, c.B, c.Dp, dtype=self.tdt)
-        self.c = mk(c.L, c.B, c.Dp, dtype=self.tdt) if keep_c else None
+        if keep_c and self.checkpointed:
+            nbytes = _lib.load().sru_amd_state_bytes(ctypes.byref(self.shape))
+            self.c = mk(nbytes // (4 * c.B * c.Dp), c.B, c.Dp, dtype=torch.float32)
+        else:
+            self.c = mk(c.L, c.B, c.Dp, dtype=self.tdt) if keep_c else None
         self.c_last = mk(c.B, c.Dp, dtype=torch.float32)
         stream = ctypes.c_void_p(torch.cuda.current_stream(self.dev).cuda_stream)
         rc = _lib.load().sru_amd_forward(

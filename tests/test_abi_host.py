@@ -23,13 +23,14 @@ def test_exports_every_declared_symbol():
 
 
 def test_struct_layout_matches_header():
-    assert ctypes.sizeof(_lib.Shape) == 48
+    assert ctypes.sizeof(_lib.Shape) == 56
     assert _lib.Shape.dirs.offset == 24 and _lib.Shape.dtype.offset == 44
+    assert _lib.Shape.state_interval.offset == 48
 
 
 def _shape(**kw):
     base = dict(length=4, batch=2, hidden=8, dirs=2, k=3, activation_type=0, skip_type=1,
-                is_custom=0, dtype=0)
+                is_custom=0, dtype=0, state_interval=0)
     base.update(kw)
     return _lib.Shape(*[base[f[0]] for f in _lib.Shape._fields_])
 
@@ -42,12 +43,15 @@ FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
     (dict(length=1 << 60), 2), (dict(dirs=3), 3), (dict(k=5), 3), (dict(k=2), 3),
     (dict(activation_type=2), 3), (dict(skip_type=3), 3), (dict(skip_type=1, k=4), 3),
     (dict(skip_type=2, k=3), 3), (dict(is_custom=2), 3), (dict(dtype=7), 4),
+    (dict(state_interval=4), 3), (dict(state_interval=8, activation_type=1), 3),
+    (dict(state_interval=8, is_custom=1), 3), (dict(state_interval=8, skip_type=0), 3),
 ])
 def test_forward_rejects_bad_shapes(kw, code):
     lib = _lib.load()
     s = _shape(**kw)
     assert lib.sru_amd_forward(ctypes.byref(s), *([FAKE] * 11), None) == code
     assert lib.sru_amd_backward_workspace_bytes(ctypes.byref(s)) == 0
+    assert lib.sru_amd_state_bytes(ctypes.byref(s)) == 0
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), 1 << 20, None) == code
 
 
@@ -70,6 +74,10 @@ def test_null_and_misaligned_pointers_and_workspace():
     assert lib.sru_amd_forward(ctypes.byref(s4), *bad, None) == 5
     need = lib.sru_amd_backward_workspace_bytes(ctypes.byref(s))
     assert need == 4 * 4 * 2 * 16
+    assert lib.sru_amd_state_bytes(ctypes.byref(s)) == 4 * 2 * 16 * 4           # (L, B, D') floats
+    assert lib.sru_amd_state_bytes(ctypes.byref(_shape(dtype=2))) == 4 * 2 * 16 * 2
+    assert lib.sru_amd_state_bytes(ctypes.byref(_shape(state_interval=8))) == 1 * 2 * 16 * 4
+    assert lib.sru_amd_state_bytes(ctypes.byref(_shape(length=33, state_interval=8, dtype=1))) == 4 * 2 * 16 * 4
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 16), None, need, None) == 6
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), need - 1, None) == 6
     bad = [FAKE] * 17

@@ -41,18 +41,26 @@ def _check_cells(name, got, ref, ref32=None):
     assert worst <= 1e-5, line
 
 
-def test_headline_shape_against_float64_oracle():
+@pytest.mark.parametrize("checkpointed", [False, True], ids=["state_every_step", "state_checkpoints"])
+def test_headline_shape_against_float64_oracle(checkpointed):
     c = Case(seed=51, scale=3 ** 0.5, zero_c0=True, **HEADLINE).f32()
-    dp = DeviceProblem(c)
+    dp = DeviceProblem(c, checkpointed=checkpointed)
     h, cs, cl = dp.forward()
     h_ref, c_ref, cl_ref = so.forward(*c.fwd_args(), **c.kw())
     print()
     _check_cells("h", to_np(h), h_ref)
-    _check_cells("c", to_np(cs), c_ref)
     _check_cells("c_last", to_np(cl), cl_ref)
-    assert _maxerr(to_np(h), h_ref) <= 1e-5 and _maxerr(to_np(cs), c_ref) <= 1e-5
+    assert _maxerr(to_np(h), h_ref) <= 1e-5
+    if checkpointed:      # rows = states after walk steps 7, 15, ...; second direction walks time backwards
+        rows = np.arange(7, c.L, 8)
+        expect = np.concatenate([c_ref[rows][..., :c.d], c_ref[c.L - 1 - rows][..., c.d:]], -1)
+        _check_cells("state checkpoints", to_np(cs), expect)
+        c_used = c_ref
+    else:
+        _check_cells("c", to_np(cs), c_ref)
+        assert _maxerr(to_np(cs), c_ref) <= 1e-5
+        c_used = to_np(cs)
     gu, gx, gwc, gb, gi = dp.backward()
-    c_used = to_np(cs)
     g_ref = so.backward(*c.fwd_args(), c_used, c.gh, c.gl, **c.kw())
     # context: the float32 serial CPU loop (the reference's own arithmetic) against the same float64 result
     g32 = so.backward(*c.fwd_args(), c_used, c.gh, c.gl, **dict(c.kw(), precision="f32"))
