@@ -216,6 +216,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": ("backward_scan_ckpt" if ckpt else "backward_scan") + " (+ reduce_partials)",
                      "achieved": bwd_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": bwd_gbs / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_GBps": None if traffic is None else traffic / (bwd_us * 1e-6) / 1e9,
                      "algorithmic_bytes_per_launch": bwd_bytes, "avg_us": bwd_us},
         "kernels": {
             "forward_scan": {"avg_us": fwd_us, "algorithmic_GBps": fwd_bytes / (fwd_us * 1e-6) / 1e9,
