@@ -1,0 +1,83 @@
+"""The entry points only enqueue kernels on the stream they are given: they can run on a
+side stream and be recorded into a HIP graph (no allocation, no memset, no host sync)."""
+import ctypes
+
+import pytest
+import torch
+
+from sru_amd import _lib, ElementwiseRecurrence
+from tests.abi import DeviceProblem
+from tests.cases import Case
+
+pytestmark = pytest.mark.gpu
+
+
+def test_side_stream_matches_default_stream():
+    c = Case(L=40, B=4, d=128, dirs=2, seed=61, pad="right", scale=1.7)
+    dp = DeviceProblem(c, checkpointed=True)
+    ref = [t.clone() for t in dp.forward()] + [t.clone() for t in dp.backward()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        got = list(dp.forward()) + list(dp.backward())
+    side.synchronize()
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+
+
+def test_forward_and_backward_replay_from_a_graph():
+    c = Case(L=33, B=4, d=128, dirs=2, seed=62, pad="right", scale=1.7, mask_c=True)
+    dp = DeviceProblem(c, checkpointed=True)
+    eager = [t.clone() for t in dp.forward(poison=False)] + [t.clone() for t in dp.backward(poison=False)]
+    torch.cuda.synchronize()
+    # static buffers: the graph replays the same pointers
+    outs = [dp.h, dp.c, dp.c_last, dp.gu, dp.gx, dp.gwc, dp.gb, dp.gi]
+    lib = _lib.load()
+    p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    nbytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(dp.shape))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.sru_amd_forward(ctypes.byref(dp.shape), p(dp.U), p(dp.x), p(dp.wc), p(dp.bias), p(dp.c0),
+                                 p(dp.mask_c), p(dp.pad), p(dp.scale), p(dp.h), p(dp.c), p(dp.c_last), stream)
+        assert rc == 0
+        rc = lib.sru_amd_backward(ctypes.byref(dp.shape), p(dp.U), p(dp.x), p(dp.wc), p(dp.bias), p(dp.c0),
+                                  p(dp.mask_c), p(dp.pad), p(dp.scale), p(dp.c), p(dp.gh), p(dp.gl),
+                                  p(dp.gu), p(dp.gx), p(dp.gwc), p(dp.gb), p(dp.gi), p(dp.ws),
+                                  ctypes.c_size_t(nbytes), stream)
+        assert rc == 0
+    for replay in range(3):
+        for t in outs:
+            t.fill_(float("nan"))          # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, outs):
+            assert torch.equal(a, b), replay
+    # new inputs in the same buffers: the replay follows them
+    dp.U.mul_(0.5)
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = [t.clone() for t in outs]
+    again = [t.clone() for t in dp.forward(poison=False)] + [t.clone() for t in dp.backward(poison=False)]
+    for a, b in zip(again, replayed):
+        assert torch.equal(a, b)
+
+
+def test_autograd_function_on_second_device_stream_and_noncontiguous_inputs():
+    c = Case(L=12, B=3, d=64, dirs=2, seed=63, scale=1.3).f32()
+    dev = "cuda:0"
+    t = lambda a: torch.tensor(a, dtype=torch.float32, device=dev)
+    u, x, wc, bias, c0 = t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0)
+    sx = torch.tensor([c.scale], device=dev)
+    h_ref, last_ref = ElementwiseRecurrence.apply(u, x, wc, bias, c0, 0, c.d, True, True, sx)
+    # U as a transposed view, x with a storage offset: the wrapper makes them contiguous / aligned
+    u_view = u.transpose(0, 1).contiguous().transpose(0, 1)
+    x_off = torch.cat([torch.zeros(1, device=dev), x.reshape(-1)])[1:].view_as(x)
+    assert not u_view.is_contiguous() and x_off.data_ptr() % 16 != 0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        h, last = ElementwiseRecurrence.apply(u_view, x_off, wc, bias, c0, 0, c.d, True, True, sx)
+    side.synchronize()
+    assert torch.equal(h, h_ref) and torch.equal(last, last_ref)
