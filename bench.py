@@ -36,6 +36,9 @@ WORKLOADS = {
     "config2": ("bi-SRU d=512 L=128 B=32 k=3, right-padded lengths in [32,128]", 128, 32, 512, 2, 3, False, True),
     "config4": ("uni-SRU d=2048 L=512 B=16 k=3", 512, 16, 2048, 1, 3, False, False),
     "config5": ("bi-SRU d=256 L=4096 B=256 k=3 forward only, lengths in [1024,4096]", 4096, 256, 256, 2, 3, True, True),
+    "config5-nopad": ("bi-SRU d=256 L=4096 B=256 k=3 forward only", 4096, 256, 256, 2, 3, True, False),
+    "headline-infer": ("bi-SRU d=1024 L=256 B=64 k=3 forward only", 256, 64, 1024, 2, 3, True, False),
+    "headline-pad": ("bi-SRU d=1024 L=256 B=64 k=3, right-padded lengths in [64,256]", 256, 64, 1024, 2, 3, False, True),
 }
 DT_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
 

@@ -37,6 +37,11 @@ namespace sru_amd {
 #define SRU_AMD_BWD_NT (kNtLoad | kNtStore)   // the same for the fast backward kernels
 #endif
 constexpr int kFwdNt = SRU_AMD_FWD_NT, kBwdNt = SRU_AMD_BWD_NT;
+// Fast forward kernels: forward_scan_chunked (1) or the ring kernel forward_scan (0). Chunked is
+// level at 2048 wavefronts and 15-30 % faster where only 256-512 wavefronts exist.
+#ifndef SRU_AMD_FWD_CHUNKED
+#define SRU_AMD_FWD_CHUNKED 1
+#endif
 template <typename T> struct Tune;
 template <> struct Tune<float> {
     static constexpr int kCols = SRU_AMD_F32_COLS, kFwdDepth = SRU_AMD_F32_FWD_DEPTH,
@@ -78,6 +83,17 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
     // what is kept for the backward pass: nothing, the state after every step, or checkpoints
     const int keep = p.ckpt ? kCkpt : (p.c ? kKeepC : 0);
     const int mode = (p.pad ? kHasPad : 0) | keep;
+#if SRU_AMD_FWD_CHUNKED
+    constexpr int TC = kCkptInterval;
+    switch (mode) {
+    case 0: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    case kHasPad: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    case kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kKeepC | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kKeepC | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    case kCkpt: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kCkpt | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    default: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kCkpt | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    }
+#endif
     switch (mode) {
     case 0: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kFwdNt, COLS, P>), grid, block, 0, st, p); break;
     case kHasPad: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kFwdNt, COLS, P>), grid, block, 0, st, p); break;

@@ -351,6 +351,132 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
 }
 
+// ================================================================= forward scan, chunked
+// Same results as forward_scan. Instead of a ring refilled step by step, the walk is cut
+// into chunks of TC steps held in two alternating register sets: the loads of chunk n+1
+// are issued in one burst before the arithmetic of chunk n, so a wavefront waits for a
+// chunk it requested a whole chunk-time earlier while the next one is already in flight.
+// (Fast kernels only; TC equals the checkpoint interval.)
+template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
+__global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p) {
+    static_assert((MODE & kGeneral) == 0, "fast kernels only");
+    static_assert(TC == kCkptInterval, "a chunk is one checkpoint interval");
+    constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
+    constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
+    constexpr bool CKPT = (MODE & kCkpt) != 0;
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
+    if (col >= p.ncols) return;
+
+    const int Dp = p.Dp;
+    const int j = (int)(col % Dp);
+    const int64_t b = col / Dp;
+    const bool flip = j >= p.d;
+
+    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], cur[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) {
+        wc1[c] = static_cast<const float *>(p.wc)[j + c];
+        wc2[c] = static_cast<const float *>(p.wc)[Dp + j + c];
+        b1[c] = p.bias[j + c];
+        b2[c] = p.bias[Dp + j + c];
+        m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
+        cur[c] = p.c0[col + c];
+    }
+    const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
+
+    const int64_t L = p.L;
+    const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + col;  // element of walk step 0
+    const int64_t es = flip ? -p.ncols : p.ncols;
+    const int64_t pf = (flip ? (L - 1) : 0) * p.B + b;
+    const int64_t ps = flip ? -p.B : p.B;
+    const T *ubase = static_cast<const T *>(p.u);
+    const T *xbase = static_cast<const T *>(p.x);
+    T *hbase = static_cast<T *>(p.h);
+    T *cbase = static_cast<T *>(p.c);
+
+    struct Chunk {
+        Group<T, COLS * K> u[TC];
+        Group<T, COLS> x[TC];
+        uint32_t pad[TC];
+    };
+
+    auto load_chunk = [&](Chunk &k, int64_t ch, int n) {
+        const int64_t s0 = ch * TC;
+#pragma unroll
+        for (int i = 0; i < TC; ++i) {
+            if (i < n) {
+                const int64_t e = ef + (s0 + i) * es;
+                k.u[i] = load_group<T, COLS * K, NTL>(ubase + e * K);
+                if (SKIP == 1) k.x[i] = load_group<T, COLS, NTL>(xbase + e);
+                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
+            }
+        }
+    };
+
+    auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) {
+        const int64_t s0 = ch * TC;
+#pragma unroll
+        for (int i = 0; i < TC; ++i) {
+            if (i < n) {
+                const bool padded = k.pad[i] != 0;
+                float hv[COLS], cv[COLS];
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) {
+                    const float u0 = k.u[i].get(c * K);
+                    const float g1 = sigmoid(k.u[i].get(c * K + 1) + wc1[c] * cur[c] + b1[c]);
+                    const float g2 = sigmoid(k.u[i].get(c * K + 2) + wc2[c] * cur[c] + b2[c]);
+                    const float cn = (cur[c] - u0) * g1 + u0;
+                    const float xv = (SKIP == 1) ? k.x[i].get(c) * sx : k.u[i].get(c * K + K - 1);
+                    const float out = (cn - xv) * m[c] * g2 + xv;
+                    cur[c] = padded ? cur[c] : cn;
+                    hv[c] = padded ? 0.0f : out;
+                    cv[c] = cur[c];
+                }
+                const int64_t e = ef + (s0 + i) * es;
+                store_group<T, COLS, NTS>(hbase + e, hv);
+                if (KEEP_C) store_group<T, COLS, NTS>(cbase + e, cv);
+            }
+        }
+        if (CKPT && n == TC) {
+#pragma unroll
+            for (int c = 0; c < COLS; ++c) p.ckpt[ch * p.ncols + col + c] = cur[c];
+        }
+    };
+
+    const int64_t nfull = L / TC;
+    const int tail = (int)(L - nfull * TC);
+    Chunk ka, kb;
+    int64_t ch = 0;
+    if (nfull > 0) load_chunk(ka, 0, TC);
+    // two chunks per iteration: every prefetch inside the loop is a real chunk
+    while (ch + 2 < nfull) {
+        load_chunk(kb, ch + 1, TC);
+        compute_chunk(ka, ch, TC);
+        __builtin_amdgcn_sched_barrier(0);
+        load_chunk(ka, ch + 2, TC);
+        compute_chunk(kb, ch + 1, TC);
+        __builtin_amdgcn_sched_barrier(0);
+        ch += 2;
+    }
+    // one or two full chunks remain (ka holds chunk ch), then the ragged tail
+    if (ch + 1 < nfull) {
+        load_chunk(kb, ch + 1, TC);
+        compute_chunk(ka, ch, TC);
+        if (tail > 0) load_chunk(ka, nfull, tail);
+        compute_chunk(kb, ch + 1, TC);
+        if (tail > 0) compute_chunk(ka, nfull, tail);
+    } else if (ch < nfull) {
+        if (tail > 0) load_chunk(kb, nfull, tail);
+        compute_chunk(ka, ch, TC);
+        if (tail > 0) compute_chunk(kb, nfull, tail);
+    } else if (tail > 0) {
+        load_chunk(kb, nfull, tail);
+        compute_chunk(kb, nfull, tail);
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
+}
+
 // ================================================================= backward scan
 // Walks each column's steps in reverse order, carrying d(loss)/d(state). The gates are
 // recomputed from U and the stored previous state. Sums of the weight_c and bias
