@@ -37,6 +37,11 @@ namespace sru_amd {
 #define SRU_AMD_BWD_NT (kNtLoad | kNtStore)   // the same for the fast backward kernels
 #endif
 constexpr int kFwdNt = SRU_AMD_FWD_NT, kBwdNt = SRU_AMD_BWD_NT;
+// 16-bit streams with few columns: below this many lanes at two columns per lane (fewer than
+// 1024 wavefronts) the kernels keep one column per lane and pair lanes for memory access.
+#ifndef SRU_AMD_PAIR_BELOW
+#define SRU_AMD_PAIR_BELOW 65536
+#endif
 // Fast forward kernels: forward_scan_chunked (1) or the ring kernel forward_scan (0). Chunked is
 // level at 2048 wavefronts and 15-30 % faster where only 256-512 wavefronts exist.
 #ifndef SRU_AMD_FWD_CHUNKED
@@ -76,7 +81,7 @@ bool pair_ok(const sru_amd_shape &s, std::initializer_list<const void *> wide,
     return true;
 }
 
-template <typename T, int K, int SKIP, int COLS>
+template <typename T, int K, int SKIP, int COLS, int PAIR = 0>
 void fast_forward(const FwdParams &p, hipStream_t st) {
     constexpr int P = Tune<T>::kFwdDepth;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
@@ -86,12 +91,12 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
 #if SRU_AMD_FWD_CHUNKED
     constexpr int TC = kCkptInterval;
     switch (mode) {
-    case 0: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
-    case kHasPad: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
-    case kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kKeepC | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
-    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kKeepC | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
-    case kCkpt: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kCkpt | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
-    default: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kCkpt | kFwdNt, COLS, TC>), grid, block, 0, st, p); return;
+    case 0: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
+    case kHasPad: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
+    case kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kKeepC | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
+    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kKeepC | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
+    case kCkpt: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kCkpt | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
+    default: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kCkpt | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
     }
 #endif
     switch (mode) {
@@ -104,13 +109,13 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
     }
 }
 
-template <typename T, int K, int SKIP, int COLS>
+template <typename T, int K, int SKIP, int COLS, int PAIR = 0>
 void fast_backward(const BwdParams &p, hipStream_t st) {
     constexpr int P = Tune<T>::kBwdDepth;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
     if (p.ckpt) {
-        if (p.pad) hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt, COLS, kCkptInterval>), grid, block, 0, st, p);
-        else hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt, COLS, kCkptInterval>), grid, block, 0, st, p);
+        if (p.pad) hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR, COLS, kCkptInterval>), grid, block, 0, st, p);
+        else hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR, COLS, kCkptInterval>), grid, block, 0, st, p);
     } else if (p.pad) {
         hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad | kBwdNt, COLS, P>), grid, block, 0, st, p);
     } else {
@@ -121,7 +126,12 @@ void fast_backward(const BwdParams &p, hipStream_t st) {
 template <typename T, int K, int SKIP>
 void pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
     if constexpr (Tune<T>::kCols == 2) {
-        if (pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c})) return fast_forward<T, K, SKIP, 2>(p, st);
+        if (pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c})) {
+#if SRU_AMD_FWD_CHUNKED
+            if (p.ncols / 2 < SRU_AMD_PAIR_BELOW) return fast_forward<T, K, SKIP, 1, kPair>(p, st);
+#endif
+            return fast_forward<T, K, SKIP, 2>(p, st);
+        }
     }
     fast_forward<T, K, SKIP, 1>(p, st);
 }
@@ -129,7 +139,10 @@ void pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
 template <typename T, int K, int SKIP>
 void pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
     if constexpr (Tune<T>::kCols == 2) {
-        if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) return fast_backward<T, K, SKIP, 2>(p, st);  // p.c is null with checkpoints
+        if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) {  // p.c is null with checkpoints
+            if (p.ckpt && p.ncols / 2 < SRU_AMD_PAIR_BELOW) return fast_backward<T, K, SKIP, 1, kPair>(p, st);
+            return fast_backward<T, K, SKIP, 2>(p, st);
+        }
     }
     fast_backward<T, K, SKIP, 1>(p, st);
 }

@@ -55,12 +55,35 @@ template <> __device__ __forceinline__ uint32_t pack_pair<bf16_bits>(float lo, f
 }
 
 // ---------------------------------------------------------------- groups of N consecutive elements
-// A Group is what one lane moves per stream and step. It is loaded and stored whole so
-// that the compiler emits one vector instruction where alignment allows, and it stays
-// in its storage form inside the ring (16-bit pairs stay packed in dwords).
+// A Group is what one lane moves per stream and step. It is loaded and stored whole, as
+// one vector of 1-4 dwords (one memory instruction), and stays in that storage form
+// inside the register ring (16-bit pairs stay packed in dwords).
 constexpr int group_align(int bytes) {
     return bytes % 16 == 0 ? 16 : bytes % 8 == 0 ? 8 : bytes % 4 == 0 ? 4 : 2;
 }
+
+// W dwords moved as one unit. Up to four they are one vector value; the vector types are
+// declared dword-aligned because a group starts wherever its column starts.
+template <int W> struct WordVec { typedef uint32_t type __attribute__((ext_vector_type(W), aligned(4))); };
+template <> struct WordVec<1> { typedef uint32_t type; };
+
+template <int W, bool VEC = (W <= 4)> struct Words;
+template <int W> struct Words<W, true> {
+    typename WordVec<W>::type v;
+    __device__ __forceinline__ uint32_t get(int i) const {
+        if constexpr (W == 1) return v;
+        else return v[i];
+    }
+    __device__ __forceinline__ void set(int i, uint32_t x) {
+        if constexpr (W == 1) v = x;
+        else v[i] = x;
+    }
+};
+template <int W> struct alignas(group_align(4 * W)) Words<W, false> {  // wider: plain dwords
+    uint32_t a[W];
+    __device__ __forceinline__ uint32_t get(int i) const { return a[i]; }
+    __device__ __forceinline__ void set(int i, uint32_t x) { a[i] = x; }
+};
 
 // storage kind: 0 float, 1 even count of 16-bit elements, 2 odd count of 16-bit elements
 template <typename T, int N> constexpr int group_kind() { return sizeof(T) == 4 ? 0 : (N % 2 == 0 ? 1 : 2); }
@@ -68,29 +91,31 @@ template <typename T, int N> constexpr int group_kind() { return sizeof(T) == 4 
 template <typename T, int N, int KIND = group_kind<T, N>()> struct Group;
 
 template <int N>
-struct alignas(group_align(4 * N)) Group<float, N, 0> {
-    float e[N];
-    __device__ __forceinline__ float get(int i) const { return e[i]; }
+struct Group<float, N, 0> {
+    static constexpr int kWords = N;
+    Words<N> w;
+    __device__ __forceinline__ float get(int i) const { return __builtin_bit_cast(float, w.get(i)); }
     __device__ __forceinline__ static Group make(const float (&v)[N]) {
         Group g;
 #pragma unroll
-        for (int i = 0; i < N; ++i) g.e[i] = v[i];
+        for (int i = 0; i < N; ++i) g.w.set(i, __builtin_bit_cast(uint32_t, v[i]));
         return g;
     }
 };
 
 // even count of 16-bit elements: dwords holding two each
 template <typename T, int N>
-struct alignas(group_align(2 * N)) Group<T, N, 1> {
-    uint32_t w[N / 2];
+struct Group<T, N, 1> {
+    static constexpr int kWords = N / 2;
+    Words<N / 2> w;
     __device__ __forceinline__ float get(int i) const {
-        return bits_to_float<T>((i & 1) ? (w[i / 2] >> 16) : (w[i / 2] & 0xffffu));
+        const uint32_t d = w.get(i / 2);
+        return bits_to_float<T>((i & 1) ? (d >> 16) : (d & 0xffffu));
     }
     __device__ __forceinline__ static Group make(const float (&v)[N]) {
         Group g;
 #pragma unroll
-        for (int i = 0; i < N / 2; ++i)
-            g.w[i] = pack_pair<T>(v[2 * i], v[2 * i + 1]);
+        for (int i = 0; i < N / 2; ++i) g.w.set(i, pack_pair<T>(v[2 * i], v[2 * i + 1]));
         return g;
     }
 };
@@ -98,6 +123,7 @@ struct alignas(group_align(2 * N)) Group<T, N, 1> {
 // odd count of 16-bit elements (one column per lane): element-wise
 template <typename T, int N>
 struct alignas(2) Group<T, N, 2> {
+    static constexpr int kWords = 0;
     uint16_t h[N];
     __device__ __forceinline__ float get(int i) const { return bits_to_float<T>(h[i]); }
     __device__ __forceinline__ static Group make(const float (&v)[N]) {
@@ -108,28 +134,17 @@ struct alignas(2) Group<T, N, 2> {
     }
 };
 
-// NT: mark the access non-temporal (streamed once; do not keep the line in the caches).
-// A group travels as 1, 2, 3 or 4 dwords; odd 16-bit groups stay ordinary accesses.
-template <int WORDS> struct Words {
-    typedef uint32_t type __attribute__((ext_vector_type(WORDS), aligned(4)));
-};
-template <> struct Words<1> { typedef uint32_t type; };
-
+// NT: mark the access non-temporal (streamed once; do not keep the line in the caches);
+// applies to groups that travel as one vector of up to four dwords.
 template <typename T, int N, bool NT = false>
 __device__ __forceinline__ Group<T, N> load_group(const T *p) {
     typedef Group<T, N> G;
-    if constexpr (NT && sizeof(G) % 4 == 0 && sizeof(G) <= 16) {
-        constexpr int W = sizeof(G) / 4;
-        typedef typename Words<W>::type vec_t;
-        const vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p));
-        uint32_t w[W];
-        if constexpr (W == 1) {
-            w[0] = v;
-        } else {
-#pragma unroll
-            for (int i = 0; i < W; ++i) w[i] = v[i];
-        }
-        return __builtin_bit_cast(G, w);
+    if constexpr (G::kWords >= 1 && G::kWords <= 4) {
+        typedef typename WordVec<G::kWords>::type vec_t;
+        G g;
+        if constexpr (NT) g.w.v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p));
+        else g.w.v = *reinterpret_cast<const vec_t *>(p);
+        return g;
     } else {
         return *reinterpret_cast<const G *>(p);
     }
@@ -137,23 +152,84 @@ __device__ __forceinline__ Group<T, N> load_group(const T *p) {
 template <typename T, int N, bool NT = false>
 __device__ __forceinline__ void store_group(T *p, const float (&v)[N]) {
     typedef Group<T, N> G;
-    if constexpr (NT && sizeof(G) % 4 == 0 && sizeof(G) <= 16) {
-        constexpr int W = sizeof(G) / 4;
-        typedef typename Words<W>::type vec_t;
-        struct Raw { uint32_t w[W]; };
-        const Raw r = __builtin_bit_cast(Raw, G::make(v));
-        vec_t out;
-        if constexpr (W == 1) {
-            out = r.w[0];
-        } else {
-#pragma unroll
-            for (int i = 0; i < W; ++i) out[i] = r.w[i];
-        }
-        __builtin_nontemporal_store(out, reinterpret_cast<vec_t *>(p));
+    const G g = G::make(v);
+    if constexpr (G::kWords >= 1 && G::kWords <= 4) {
+        typedef typename WordVec<G::kWords>::type vec_t;
+        if constexpr (NT) __builtin_nontemporal_store(g.w.v, reinterpret_cast<vec_t *>(p));
+        else *reinterpret_cast<vec_t *>(p) = g.w.v;
     } else {
-        *reinterpret_cast<G *>(p) = G::make(v);
+        *reinterpret_cast<G *>(p) = g;
     }
 }
+
+// ---------------------------------------------------------------- a lane's share of a stream
+// What one lane moves per stream and step (N elements per column), and how it finds its
+// own elements in it.
+//   plain: the lane's COLS columns form one Group<T, COLS*N> at the lane's own element.
+//   PAIR (16-bit elements, one column per lane): lanes 2i and 2i+1 own adjacent columns
+//   whose N+N elements form one dword-granular group. Both lanes load that group (same
+//   address: the hardware serves the pair with one fetch) and each picks its half; for a
+//   store the even lane takes the odd lane's values through a DPP lane swap and writes the
+//   group, the odd lane writes nothing. This keeps one column per lane (twice the
+//   wavefronts of COLS = 2, which matters when columns are few) with the same dword-wide
+//   memory instructions.
+template <typename T, int N, int COLS, bool PAIR>
+struct Stream {
+    static_assert(!PAIR || (COLS == 1 && sizeof(T) == 2), "pairs are for 16-bit elements, one column per lane");
+    static constexpr int kElems = (PAIR ? 2 : COLS) * N;
+    using G = Group<T, kElems>;
+
+    // e: element index of the lane's first own element (in units of columns); q: lane parity
+    template <bool NT>
+    __device__ __forceinline__ static G load(const T *base, int64_t e, int q) {
+        return load_group<T, kElems, NT>(base + (e - (PAIR ? q : 0)) * N);
+    }
+    // all elements of the lane's columns as floats: out[c * N + i] = element i of column c
+    __device__ __forceinline__ static void unpack(const G &g, int q, float (&out)[COLS * N]) {
+        if constexpr (!PAIR) {
+#pragma unroll
+            for (int i = 0; i < COLS * N; ++i) out[i] = g.get(i);
+        } else {
+            // The pair's group holds the even lane's N elements, then the odd lane's. Whole-dword
+            // selects and one funnel shift move the lane's own elements to the front (a select
+            // between g.get(i) and g.get(N + i) would become a run-time vector index).
+            const uint32_t sh = (N % 2) ? 16u * (uint32_t)q : 0u;  // odd N: the odd lane starts mid-dword
+            constexpr int W = (N + 1) / 2;                         // dwords holding the lane's elements
+            uint32_t own[W];
+            if constexpr (N % 2 == 0) {
+#pragma unroll
+                for (int i = 0; i < W; ++i) own[i] = q ? g.w.get(W + i) : g.w.get(i);
+            } else if constexpr (N == 1) {
+                own[0] = g.w.get(0) >> sh;
+            } else {
+                static_assert(N == 3, "odd groups are 1 or 3 elements");
+                const uint32_t a = q ? g.w.get(1) : g.w.get(0);
+                const uint32_t b = q ? g.w.get(2) : g.w.get(1);
+                own[0] = __builtin_amdgcn_alignbit(b, a, sh);
+                own[1] = b >> sh;
+            }
+#pragma unroll
+            for (int i = 0; i < N; ++i)
+                out[i] = bits_to_float<T>((i & 1) ? (own[i / 2] >> 16) : (own[i / 2] & 0xffffu));
+        }
+    }
+    template <bool NT>
+    __device__ __forceinline__ static void store(T *base, int64_t e, int q, const float (&v)[COLS * N]) {
+        if constexpr (PAIR) {
+            float both[2 * N];
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                both[i] = v[i];
+                // quad_perm [1,0,3,2]: the value of the neighbouring lane of the pair
+                both[N + i] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                    0, __builtin_bit_cast(int, v[i]), 0xB1, 0xf, 0xf, false));
+            }
+            if (q == 0) store_group<T, kElems, NT>(base + e * N, both);
+        } else {
+            store_group<T, kElems, NT>(base + e * N, v);
+        }
+    }
+};
 
 // ---------------------------------------------------------------- gate arithmetic
 // sigmoid through the hardware exp2 and reciprocal (1 ulp each): absolute error of the
@@ -204,6 +280,7 @@ constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
 constexpr int kNtLoad = 8;   // MODE bit: stream loads are non-temporal
 constexpr int kNtStore = 16; // MODE bit: stream stores are non-temporal
 constexpr int kCkpt = 32;    // MODE bit (fast forward kernels): store a state checkpoint per chunk
+constexpr int kPair = 64;    // MODE bit (chunked fast kernels, 16-bit): lanes pair up for memory access
 
 // Checkpointed state. Instead of the state after every step (4 bytes per cell written by
 // the forward pass and read again by the backward pass), the forward pass can keep only
@@ -356,16 +433,21 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
 // into chunks of TC steps held in two alternating register sets: the loads of chunk n+1
 // are issued in one burst before the arithmetic of chunk n, so a wavefront waits for a
 // chunk it requested a whole chunk-time earlier while the next one is already in flight.
-// (Fast kernels only; TC equals the checkpoint interval.)
+// (Fast kernels only; TC equals the checkpoint interval. The two lambdas must be inlined at
+// every call site: a chunk that is passed by reference to a real function lives in scratch
+// memory instead of registers.)
 template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
 __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     static_assert(TC == kCkptInterval, "a chunk is one checkpoint interval");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
-    constexpr bool CKPT = (MODE & kCkpt) != 0;
+    constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0;
+    using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
+    using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
+    const int q = PAIR ? (int)(threadIdx.x & 1) : 0;  // columns of a pair are col - q, col - q + 1
 
     const int Dp = p.Dp;
     const int j = (int)(col % Dp);
@@ -395,46 +477,48 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     T *cbase = static_cast<T *>(p.c);
 
     struct Chunk {
-        Group<T, COLS * K> u[TC];
-        Group<T, COLS> x[TC];
+        typename SU::G u[TC];
+        typename S1::G x[TC];
         uint32_t pad[TC];
     };
 
-    auto load_chunk = [&](Chunk &k, int64_t ch, int n) {
+    auto load_chunk = [&](Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
         const int64_t s0 = ch * TC;
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const int64_t e = ef + (s0 + i) * es;
-                k.u[i] = load_group<T, COLS * K, NTL>(ubase + e * K);
-                if (SKIP == 1) k.x[i] = load_group<T, COLS, NTL>(xbase + e);
+                k.u[i] = SU::template load<NTL>(ubase, e, q);
+                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase, e, q);
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
     };
 
-    auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) {
+    auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
         const int64_t s0 = ch * TC;
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const bool padded = k.pad[i] != 0;
-                float hv[COLS], cv[COLS];
+                float hv[COLS], cv[COLS], uu[COLS * K], xx[COLS] = {};
+                SU::unpack(k.u[i], q, uu);
+                if (SKIP == 1) S1::unpack(k.x[i], q, xx);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
-                    const float u0 = k.u[i].get(c * K);
-                    const float g1 = sigmoid(k.u[i].get(c * K + 1) + wc1[c] * cur[c] + b1[c]);
-                    const float g2 = sigmoid(k.u[i].get(c * K + 2) + wc2[c] * cur[c] + b2[c]);
+                    const float u0 = uu[c * K];
+                    const float g1 = sigmoid(uu[c * K + 1] + wc1[c] * cur[c] + b1[c]);
+                    const float g2 = sigmoid(uu[c * K + 2] + wc2[c] * cur[c] + b2[c]);
                     const float cn = (cur[c] - u0) * g1 + u0;
-                    const float xv = (SKIP == 1) ? k.x[i].get(c) * sx : k.u[i].get(c * K + K - 1);
+                    const float xv = (SKIP == 1) ? xx[c] * sx : uu[c * K + K - 1];
                     const float out = (cn - xv) * m[c] * g2 + xv;
                     cur[c] = padded ? cur[c] : cn;
                     hv[c] = padded ? 0.0f : out;
                     cv[c] = cur[c];
                 }
                 const int64_t e = ef + (s0 + i) * es;
-                store_group<T, COLS, NTS>(hbase + e, hv);
-                if (KEEP_C) store_group<T, COLS, NTS>(cbase + e, cv);
+                S1::template store<NTS>(hbase, e, q, hv);
+                if (KEEP_C) S1::template store<NTS>(cbase, e, q, cv);
             }
         }
         if (CKPT && n == TC) {
@@ -664,9 +748,12 @@ template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
 __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
-    constexpr bool HAS_PAD = (MODE & kHasPad) != 0;
+    constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0;
+    using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
+    using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
+    const int q = PAIR ? (int)(threadIdx.x & 1) : 0;
 
     const int Dp = p.Dp;
     const int j = (int)(col % Dp);
@@ -702,23 +789,23 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     T *gxbase = static_cast<T *>(p.gx);
 
     struct Chunk {
-        Group<T, COLS * K> u[TC];
-        Group<T, COLS> x[TC];
-        Group<T, COLS> gh[TC];
+        typename SU::G u[TC];
+        typename S1::G x[TC];
+        typename S1::G gh[TC];
         uint32_t pad[TC];
         float cstart[COLS];  // state before the chunk's first step
     };
 
     // n: number of valid steps in the chunk (TC except for a ragged last chunk)
-    auto load_chunk = [&](Chunk &k, int64_t ch, int n) {
+    auto load_chunk = [&](Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
         const int64_t s0 = ch * TC;
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const int64_t e = ef + (s0 + i) * es;
-                k.u[i] = load_group<T, COLS * K, NTL>(ubase + e * K);
-                if (SKIP == 1) k.x[i] = load_group<T, COLS, NTL>(xbase + e);
-                k.gh[i] = load_group<T, COLS, NTL>(ghbase + e);
+                k.u[i] = SU::template load<NTL>(ubase, e, q);
+                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase, e, q);
+                k.gh[i] = S1::template load<NTL>(ghbase, e, q);
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
@@ -727,23 +814,27 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
             k.cstart[c] = (ch == 0) ? c_init[c] : p.ckpt[(ch - 1) * p.ncols + col + c];
     };
 
-    auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) {
+    auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
         const int64_t s0 = ch * TC;
         float st[TC + 1][COLS];  // st[i] = state before step i of the chunk
         float g1[TC][COLS], g2[TC][COLS];
+        float u0s[TC][COLS], xs[TC][COLS];  // candidate stream and (k = 4) skip stream, decoded once
 #pragma unroll
         for (int c = 0; c < COLS; ++c) st[0][c] = k.cstart[c];
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const bool padded = k.pad[i] != 0;
+                float uu[COLS * K];
+                SU::unpack(k.u[i], q, uu);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float cp = st[i][c];
-                    const float u0 = k.u[i].get(c * K);
-                    g1[i][c] = sigmoid(k.u[i].get(c * K + 1) + wc1[c] * cp + b1[c]);
-                    g2[i][c] = sigmoid(k.u[i].get(c * K + 2) + wc2[c] * cp + b2[c]);
-                    const float cn = (cp - u0) * g1[i][c] + u0;
+                    u0s[i][c] = uu[c * K];
+                    if (SKIP == 2) xs[i][c] = uu[c * K + K - 1];
+                    g1[i][c] = sigmoid(uu[c * K + 1] + wc1[c] * cp + b1[c]);
+                    g2[i][c] = sigmoid(uu[c * K + 2] + wc2[c] * cp + b2[c]);
+                    const float cn = (cp - u0s[i][c]) * g1[i][c] + u0s[i][c];
                     st[i + 1][c] = padded ? cp : cn;
                 }
             }
@@ -752,14 +843,16 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         for (int i = TC - 1; i >= 0; --i) {
             if (i < n) {
                 const bool padded = k.pad[i] != 0;
-                float gu[COLS * K], gx[COLS];
+                float gu[COLS * K], gx[COLS], xx[COLS] = {}, ghs[COLS];
+                if (SKIP == 1) S1::unpack(k.x[i], q, xx);
+                S1::unpack(k.gh[i], q, ghs);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float cp = st[i][c], val = st[i + 1][c];
-                    const float u0 = k.u[i].get(c * K);
+                    const float u0 = u0s[i][c];
                     const float G1 = g1[i][c], G2 = g2[i][c];
-                    const float xv = (SKIP == 1) ? k.x[i].get(c) * sx : k.u[i].get(c * K + K - 1);
-                    const float gh = k.gh[i].get(c);
+                    const float xv = (SKIP == 1) ? xx[c] * sx : xs[i][c];
+                    const float gh = ghs[c];
 
                     const float gg2 = gh * (val - xv) * m[c] * (G2 * (1.0f - G2));
                     const float gc = gh * m[c] * G2 + cur[c];
@@ -779,8 +872,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                     cur[c] = padded ? cur[c] : ncur;
                 }
                 const int64_t e = ef + (s0 + i) * es;
-                store_group<T, COLS * K, NTS>(gubase + e * K, gu);
-                if (SKIP == 1) store_group<T, COLS, NTS>(gxbase + e, gx);
+                SU::template store<NTS>(gubase, e, q, gu);
+                if (SKIP == 1) S1::template store<NTS>(gxbase, e, q, gx);
             }
         }
     };

@@ -75,6 +75,23 @@ def test_headline_shape_against_float64_oracle(checkpointed):
     assert e_b <= 1e-5 * max(1.0, np.abs(g_ref[3]).max())
 
 
+@pytest.mark.parametrize("checkpointed", [False, True], ids=["state_every_step", "state_checkpoints"])
+def test_headline_shape_bf16_streams(checkpointed):
+    # the two-columns-per-lane kernels (16-bit streams, 65 536 lanes); tolerance 2e-2 * max(1, max|ref|)
+    c = Case(seed=55, scale=3 ** 0.5, pad="right", **HEADLINE)
+    dp = DeviceProblem(c, "bf16", checkpointed=checkpointed)
+    rc = dp.rounded_case()
+    h, cs, cl = dp.forward()
+    h_ref, c_ref, cl_ref = so.forward(*rc.fwd_args(), **rc.kw())
+    rel = lambda got, ref: _maxerr(got, ref) / max(1.0, float(np.abs(ref).max()))
+    assert rel(to_np(h), h_ref) <= 2e-2 and rel(to_np(cl), cl_ref) <= 1e-3
+    gu, gx, gwc, gb, gi = dp.backward()
+    c_used = c_ref if checkpointed else to_np(cs)
+    g_ref = so.backward(*rc.fwd_args(), c_used, rc.gh, rc.gl, **rc.kw())
+    for got, ref in zip((gu, gx, gwc, gb, gi), g_ref):
+        assert rel(to_np(got), ref) <= 2e-2
+
+
 def _device_case(seed=52, **over):
     kw = dict(HEADLINE, seed=seed, scale=3 ** 0.5, pad="right", mask_c=True)
     kw.update(over)
