@@ -1,5 +1,7 @@
 """Builds sru_amd/libsru_amd.so for gfx950 with hipcc.  `python -m sru_amd.build`"""
+import json
 import os
+import re
 import subprocess
 import sys
 
@@ -18,17 +20,45 @@ HIPCC_FLAGS = [
 ]
 
 
+# A kernel whose register ring or chunk ends up in scratch memory runs several times slower
+# with unchanged results, so the build checks the compiler's resource report and refuses
+# more than a few spilled dwords per lane.
+MAX_SCRATCH_BYTES = 64
+_REMARK = re.compile(r"remark: .*?(Function Name: (?P<name>\S+)|ScratchSize \[bytes/lane\]: (?P<scratch>\d+)"
+                     r"|VGPRs: (?P<vgprs>\d+))")
+
+
 def _run(cmd, verbose):
+    """Runs one hipcc command; returns {kernel: (vgprs, scratch_bytes)} from its resource remarks."""
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    # the host pass does not know the device-only target feature and says so: harmless
-    out = "\n".join(l for l in proc.stdout.splitlines()
-                    if "packed-fp32-ops" not in l and l.strip())
-    if out and (verbose or proc.returncode):
-        print(out, flush=True)
+    usage, name, vgprs = {}, None, None
+    other = []
+    in_remark = False
+    for line in proc.stdout.splitlines():
+        if in_remark and re.match(r"\s*(\d+)?\s*\|", line):
+            continue            # source excerpt under a remark
+        in_remark = "remark:" in line
+        m = _REMARK.search(line)
+        if m:
+            if m.group("name"):
+                name, vgprs = m.group("name"), None
+            elif m.group("vgprs") and " VGPRs:" in line:
+                vgprs = int(m.group("vgprs"))
+            elif m.group("scratch") is not None and name:
+                usage[name] = (vgprs, int(m.group("scratch")))
+            continue
+        # the host pass does not know the device-only target feature and says so: harmless
+        if ("remark:" in line or "packed-fp32-ops" in line or not line.strip()
+                or line.startswith("In file included from")):
+            continue
+        other.append(line)
+    if other and (verbose or proc.returncode):
+        print("\n".join(other), flush=True)
     if proc.returncode:
         raise RuntimeError("hipcc failed: " + " ".join(cmd))
+    return usage
 
 
 def build(verbose=True, output=OUTPUT, defines=()):
@@ -42,9 +72,21 @@ def build(verbose=True, output=OUTPUT, defines=()):
     os.makedirs(obj_dir, exist_ok=True)
     objs = [os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o") for src in SOURCES]
     extra = ["-D" + d for d in defines]
-    jobs = [[hipcc] + HIPCC_FLAGS + extra + ["-c", src, "-o", obj] for src, obj in zip(SOURCES, objs)]
+    jobs = [[hipcc] + HIPCC_FLAGS + extra + ["-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
+            for src, obj in zip(SOURCES, objs)]
+    usage = {}
     with ThreadPoolExecutor(max_workers=4) as pool:
-        list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
+        for part in pool.map(lambda cmd: _run(cmd, verbose), jobs):
+            usage.update(part)
+    with open(os.path.join(obj_dir, "resource_usage.json"), "w") as f:
+        json.dump({k: {"vgprs": v[0], "scratch_bytes": v[1]} for k, v in sorted(usage.items())}, f, indent=1)
+    spilled = {k: v[1] for k, v in usage.items() if v[1] > MAX_SCRATCH_BYTES}
+    if spilled:
+        raise RuntimeError(f"{len(spilled)} kernels keep more than {MAX_SCRATCH_BYTES} bytes per lane in "
+                           f"scratch memory, e.g. {sorted(spilled.items(), key=lambda kv: -kv[1])[:3]}")
+    if verbose:
+        print(f"{len(usage)} kernels, largest scratch {max([v[1] for v in usage.values()] or [0])} bytes/lane, "
+              f"largest VGPR count {max([v[0] or 0 for v in usage.values()] or [0])}", flush=True)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", output], verbose)
     return output
 

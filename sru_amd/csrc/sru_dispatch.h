@@ -98,7 +98,8 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
     case kCkpt: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kCkpt | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
     default: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kCkpt | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
     }
-#endif
+#else
+    static_assert(PAIR == 0, "lane pairing exists in the chunked kernels only");
     switch (mode) {
     case 0: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kFwdNt, COLS, P>), grid, block, 0, st, p); break;
     case kHasPad: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
@@ -107,6 +108,7 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
     case kCkpt: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kCkpt | kFwdNt, COLS, kCkptInterval>), grid, block, 0, st, p); break;
     default: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kCkpt | kFwdNt, COLS, kCkptInterval>), grid, block, 0, st, p); break;
     }
+#endif
 }
 
 template <typename T, int K, int SKIP, int COLS, int PAIR = 0>

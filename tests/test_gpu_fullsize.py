@@ -169,3 +169,44 @@ def test_long_sequence_inference_shape_fp16():
     h_ref, _, cl_ref = so.forward(*rc.fwd_args(), **rc.kw())
     assert _maxerr(to_np(h), h_ref) <= 2e-2 * max(1.0, np.abs(h_ref).max())
     assert _maxerr(to_np(cl), cl_ref) <= 1e-3 * max(1.0, np.abs(cl_ref).max())
+
+
+def test_offsets_beyond_32_bits_long_sequence_k4():
+    # config-5 scale with k=4: U has exactly 2^31 elements (4.3 GB in float16), so element and
+    # byte offsets leave the 32-bit range. Checked through batch independence: the first and the
+    # last batch row of the big run must equal a run on those two rows alone, bit for bit.
+    import ctypes
+    from sru_amd import _lib
+    L, B, d, dirs, k = 4096, 256, 256, 2, 4
+    Dp = d * dirs
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(77)
+    U = torch.empty(L, B, Dp * k, dtype=torch.float16, device=dev)
+    for t0 in range(0, L, 512):
+        U[t0:t0 + 512] = torch.randn(512, B, Dp * k, device=dev, generator=g).half()
+    assert U.numel() == 2 ** 31
+    wc = (torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1)
+    bias = torch.randn(2 * Dp, device=dev, generator=g) * 0.3
+    c0 = torch.randn(B, Dp, device=dev, generator=g)
+    lens = torch.randint(1024, L + 1, (B,), device=dev, generator=g)
+    pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :])
+    lib = _lib.load()
+    p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+
+    def run(U_, c0_, pad_, batch):
+        shape = _lib.Shape(L, batch, d, dirs, k, 0, 2, 0, _lib.F16, 1)
+        h = torch.full((L, batch, Dp), float("nan"), dtype=torch.float16, device=dev)
+        cl = torch.full((batch, Dp), float("nan"), device=dev)
+        padb = pad_.contiguous().view(torch.uint8)
+        rc = lib.sru_amd_forward(ctypes.byref(shape), p(U_), None, p(wc), p(bias), p(c0_), None, p(padb),
+                                 None, p(h), None, p(cl), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, _lib.status_string(rc)
+        torch.cuda.synchronize()
+        return h, cl
+
+    h_big, cl_big = run(U, c0, pad, B)
+    assert not torch.isnan(h_big[-1]).any() and not torch.isnan(h_big[0]).any()
+    rows = torch.tensor([0, B - 1], device=dev)
+    h_small, cl_small = run(U[:, rows].contiguous(), c0[rows].contiguous(), pad[:, rows], 2)
+    assert torch.equal(h_big[:, rows], h_small) and torch.equal(cl_big[rows], cl_small)
+    assert float(h_big[pad].abs().max()) == 0.0
