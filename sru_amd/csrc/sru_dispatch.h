@@ -81,8 +81,21 @@ bool pair_ok(const sru_amd_shape &s, std::initializer_list<const void *> wide,
     return true;
 }
 
-template <typename T, int K, int SKIP, int COLS, int PAIR = 0>
+// true when every wavefront lies inside one direction and one batch row
+#ifndef SRU_AMD_UNIFORM
+#define SRU_AMD_UNIFORM 1   // 0: never use the scalar-addressing builds (tuning)
+#endif
+inline bool wave_uniform(int32_t d, int cols) { return SRU_AMD_UNIFORM && d % (kBlock * cols) == 0; }
+
+template <typename T, int K, int SKIP, int COLS, int PAIR = 0, int UNI = -1>
 void fast_forward(const FwdParams &p, hipStream_t st) {
+#if SRU_AMD_FWD_CHUNKED
+    if constexpr (UNI < 0) {   // pick the scalar-addressing build of the kernel when the shape allows
+        if (wave_uniform(p.d, COLS)) return fast_forward<T, K, SKIP, COLS, PAIR, kUniform>(p, st);
+        return fast_forward<T, K, SKIP, COLS, PAIR, 0>(p, st);
+    }
+#endif
+    constexpr int X = PAIR | (UNI > 0 ? UNI : 0);
     constexpr int P = Tune<T>::kFwdDepth;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
     // what is kept for the backward pass: nothing, the state after every step, or checkpoints
@@ -91,12 +104,12 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
 #if SRU_AMD_FWD_CHUNKED
     constexpr int TC = kCkptInterval;
     switch (mode) {
-    case 0: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
-    case kHasPad: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
-    case kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kKeepC | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
-    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kKeepC | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
-    case kCkpt: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kCkpt | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
-    default: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kCkpt | kFwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); return;
+    case 0: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kFwdNt | X, COLS, TC>), grid, block, 0, st, p); return;
+    case kHasPad: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kFwdNt | X, COLS, TC>), grid, block, 0, st, p); return;
+    case kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kKeepC | kFwdNt | X, COLS, TC>), grid, block, 0, st, p); return;
+    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kKeepC | kFwdNt | X, COLS, TC>), grid, block, 0, st, p); return;
+    case kCkpt: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kCkpt | kFwdNt | X, COLS, TC>), grid, block, 0, st, p); return;
+    default: hipLaunchKernelGGL((forward_scan_chunked<T, K, SKIP, kHasPad | kCkpt | kFwdNt | X, COLS, TC>), grid, block, 0, st, p); return;
     }
 #else
     static_assert(PAIR == 0, "lane pairing exists in the chunked kernels only");
@@ -114,10 +127,16 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
 template <typename T, int K, int SKIP, int COLS, int PAIR = 0>
 void fast_backward(const BwdParams &p, hipStream_t st) {
     constexpr int P = Tune<T>::kBwdDepth;
+    constexpr int TC = kCkptInterval;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
     if (p.ckpt) {
-        if (p.pad) hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR, COLS, kCkptInterval>), grid, block, 0, st, p);
-        else hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR, COLS, kCkptInterval>), grid, block, 0, st, p);
+        const int mode = (p.pad ? 1 : 0) | (wave_uniform(p.d, COLS) ? 2 : 0);
+        switch (mode) {
+        case 0: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); break;
+        case 1: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); break;
+        case 2: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR | kUniform, COLS, TC>), grid, block, 0, st, p); break;
+        default: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR | kUniform, COLS, TC>), grid, block, 0, st, p); break;
+        }
     } else if (p.pad) {
         hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad | kBwdNt, COLS, P>), grid, block, 0, st, p);
     } else {

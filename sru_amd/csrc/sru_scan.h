@@ -179,10 +179,14 @@ struct Stream {
     static constexpr int kElems = (PAIR ? 2 : COLS) * N;
     using G = Group<T, kElems>;
 
-    // e: element index of the lane's first own element (in units of columns); q: lane parity
+    // row: pointer to the stream's elements of the wavefront's (or lane's) first column at this
+    // step; lane: the lane's column offset from there; q: lane parity
+    // (signed arithmetic: with per-lane row pointers lane is 0 and the odd lane of a pair
+    // steps back to the even lane's column)
     template <bool NT>
-    __device__ __forceinline__ static G load(const T *base, int64_t e, int q) {
-        return load_group<T, kElems, NT>(base + (e - (PAIR ? q : 0)) * N);
+    __device__ __forceinline__ static G load(const T *row, uint32_t lane, int q) {
+        const int32_t first = (int32_t)lane - (PAIR ? q : 0);
+        return load_group<T, kElems, NT>(row + first * N);
     }
     // all elements of the lane's columns as floats: out[c * N + i] = element i of column c
     __device__ __forceinline__ static void unpack(const G &g, int q, float (&out)[COLS * N]) {
@@ -214,7 +218,7 @@ struct Stream {
         }
     }
     template <bool NT>
-    __device__ __forceinline__ static void store(T *base, int64_t e, int q, const float (&v)[COLS * N]) {
+    __device__ __forceinline__ static void store(T *row, uint32_t lane, int q, const float (&v)[COLS * N]) {
         if constexpr (PAIR) {
             float both[2 * N];
 #pragma unroll
@@ -224,9 +228,9 @@ struct Stream {
                 both[N + i] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
                     0, __builtin_bit_cast(int, v[i]), 0xB1, 0xf, 0xf, false));
             }
-            if (q == 0) store_group<T, kElems, NT>(base + e * N, both);
+            if (q == 0) store_group<T, kElems, NT>(row + (int32_t)lane * N, both);
         } else {
-            store_group<T, kElems, NT>(base + e * N, v);
+            store_group<T, kElems, NT>(row + (int32_t)lane * N, v);
         }
     }
 };
@@ -281,6 +285,9 @@ constexpr int kNtLoad = 8;   // MODE bit: stream loads are non-temporal
 constexpr int kNtStore = 16; // MODE bit: stream stores are non-temporal
 constexpr int kCkpt = 32;    // MODE bit (fast forward kernels): store a state checkpoint per chunk
 constexpr int kPair = 64;    // MODE bit (chunked fast kernels, 16-bit): lanes pair up for memory access
+constexpr int kUniform = 128;// MODE bit (chunked fast kernels): a wavefront lies inside one direction and
+                             // one batch row (d is a multiple of 64 * COLS), so the time index, the row
+                             // pointers and the padding flag are scalar: no per-lane address arithmetic
 
 // Checkpointed state. Instead of the state after every step (4 bytes per cell written by
 // the forward pass and read again by the backward pass), the forward pass can keep only
@@ -442,17 +449,21 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     static_assert(TC == kCkptInterval, "a chunk is one checkpoint interval");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
-    constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0;
+    constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;  // columns of a pair are col - q, col - q + 1
 
+    // colu decides direction and batch row: the wavefront's first column when that is the same
+    // for all its lanes (scalar), else the lane's own column
+    const int64_t colu = UNI ? (int64_t)blockIdx.x * (kBlock * COLS) : col;
+    const uint32_t lane = (uint32_t)(col - colu);
     const int Dp = p.Dp;
-    const int j = (int)(col % Dp);
-    const int64_t b = col / Dp;
-    const bool flip = j >= p.d;
+    const int ju = (int)(colu % Dp);
+    const int j = ju + (int)lane;
+    const bool flip = ju >= p.d;
 
     float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], cur[COLS];
 #pragma unroll
@@ -467,9 +478,11 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
 
     const int64_t L = p.L;
-    const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + col;  // element of walk step 0
+    const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + colu;  // element of walk step 0 (column colu)
     const int64_t es = flip ? -p.ncols : p.ncols;
-    const int64_t pf = (flip ? (L - 1) : 0) * p.B + b;
+    // per-lane on purpose: with a scalar address the padding bytes would come through the
+    // scalar data cache, whose loads cannot be pipelined behind the vector loads
+    const int64_t pf = (flip ? (L - 1) : 0) * p.B + col / Dp;
     const int64_t ps = flip ? -p.B : p.B;
     const T *ubase = static_cast<const T *>(p.u);
     const T *xbase = static_cast<const T *>(p.x);
@@ -488,8 +501,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const int64_t e = ef + (s0 + i) * es;
-                k.u[i] = SU::template load<NTL>(ubase, e, q);
-                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase, e, q);
+                k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
+                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
@@ -517,8 +530,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
                     cv[c] = cur[c];
                 }
                 const int64_t e = ef + (s0 + i) * es;
-                S1::template store<NTS>(hbase, e, q, hv);
-                if (KEEP_C) S1::template store<NTS>(cbase, e, q, cv);
+                S1::template store<NTS>(hbase + e, lane, q, hv);
+                if (KEEP_C) S1::template store<NTS>(cbase + e, lane, q, cv);
             }
         }
         if (CKPT && n == TC) {
@@ -535,9 +548,11 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     // two chunks per iteration: every prefetch inside the loop is a real chunk
     while (ch + 2 < nfull) {
         load_chunk(kb, ch + 1, TC);
+        __builtin_amdgcn_sched_barrier(0);  // all loads of the next chunk first, then the arithmetic
         compute_chunk(ka, ch, TC);
         __builtin_amdgcn_sched_barrier(0);
         load_chunk(ka, ch + 2, TC);
+        __builtin_amdgcn_sched_barrier(0);
         compute_chunk(kb, ch + 1, TC);
         __builtin_amdgcn_sched_barrier(0);
         ch += 2;
@@ -748,17 +763,19 @@ template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
 __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
-    constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0;
+    constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;
 
+    const int64_t colu = UNI ? (int64_t)blockIdx.x * (kBlock * COLS) : col;  // see forward_scan_chunked
+    const uint32_t lane = (uint32_t)(col - colu);
     const int Dp = p.Dp;
-    const int j = (int)(col % Dp);
-    const int64_t b = col / Dp;
-    const bool flip = j >= p.d;
+    const int ju = (int)(colu % Dp);
+    const int j = ju + (int)lane;
+    const bool flip = ju >= p.d;
 
     float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
     float cur[COLS];  // d loss / d state
@@ -778,9 +795,11 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
 
     const int64_t L = p.L;
     // forward-walk step s of this column sits at element ef + s * es
-    const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + col;
+    const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + colu;
     const int64_t es = flip ? -p.ncols : p.ncols;
-    const int64_t pf = (flip ? (L - 1) : 0) * p.B + b;
+    // per-lane on purpose: with a scalar address the padding bytes would come through the
+    // scalar data cache, whose loads cannot be pipelined behind the vector loads
+    const int64_t pf = (flip ? (L - 1) : 0) * p.B + col / Dp;
     const int64_t ps = flip ? -p.B : p.B;
     const T *ubase = static_cast<const T *>(p.u);
     const T *xbase = static_cast<const T *>(p.x);
@@ -803,9 +822,9 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const int64_t e = ef + (s0 + i) * es;
-                k.u[i] = SU::template load<NTL>(ubase, e, q);
-                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase, e, q);
-                k.gh[i] = S1::template load<NTL>(ghbase, e, q);
+                k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
+                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
+                k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
@@ -872,8 +891,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                     cur[c] = padded ? cur[c] : ncur;
                 }
                 const int64_t e = ef + (s0 + i) * es;
-                SU::template store<NTS>(gubase, e, q, gu);
-                if (SKIP == 1) S1::template store<NTS>(gxbase, e, q, gx);
+                SU::template store<NTS>(gubase + e * K, lane, q, gu);
+                if (SKIP == 1) S1::template store<NTS>(gxbase + e, lane, q, gx);
             }
         }
     };
