@@ -149,7 +149,9 @@ void pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
     if constexpr (Tune<T>::kCols == 2) {
         if (pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c})) {
 #if SRU_AMD_FWD_CHUNKED
-            if (p.ncols / 2 < SRU_AMD_PAIR_BELOW) return fast_forward<T, K, SKIP, 1, kPair>(p, st);
+            if constexpr (sizeof(T) == 2) {
+                if (p.ncols / 2 < SRU_AMD_PAIR_BELOW) return fast_forward<T, K, SKIP, 1, kPair>(p, st);
+            }
 #endif
             return fast_forward<T, K, SKIP, 2>(p, st);
         }
@@ -161,7 +163,9 @@ template <typename T, int K, int SKIP>
 void pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
     if constexpr (Tune<T>::kCols == 2) {
         if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) {  // p.c is null with checkpoints
-            if (p.ckpt && p.ncols / 2 < SRU_AMD_PAIR_BELOW) return fast_backward<T, K, SKIP, 1, kPair>(p, st);
+            if constexpr (sizeof(T) == 2) {
+                if (p.ckpt && p.ncols / 2 < SRU_AMD_PAIR_BELOW) return fast_backward<T, K, SKIP, 1, kPair>(p, st);
+            }
             return fast_backward<T, K, SKIP, 2>(p, st);
         }
     }

@@ -79,10 +79,14 @@ template <int W> struct Words<W, true> {
         else v[i] = x;
     }
 };
-template <int W> struct alignas(group_align(4 * W)) Words<W, false> {  // wider: plain dwords
-    uint32_t a[W];
-    __device__ __forceinline__ uint32_t get(int i) const { return a[i]; }
-    __device__ __forceinline__ void set(int i, uint32_t x) { a[i] = x; }
+template <int W> struct Words<W, false> {  // 6 or 8 dwords: two vectors of 3 or 4
+    static_assert(W == 6 || W == 8, "wide groups are two vectors");
+    typename WordVec<W / 2>::type lo, hi;
+    __device__ __forceinline__ uint32_t get(int i) const { return i < W / 2 ? lo[i] : hi[i - W / 2]; }
+    __device__ __forceinline__ void set(int i, uint32_t x) {
+        if (i < W / 2) lo[i] = x;
+        else hi[i - W / 2] = x;
+    }
 };
 
 // storage kind: 0 float, 1 even count of 16-bit elements, 2 odd count of 16-bit elements
@@ -135,15 +139,28 @@ struct alignas(2) Group<T, N, 2> {
 };
 
 // NT: mark the access non-temporal (streamed once; do not keep the line in the caches);
-// applies to groups that travel as one vector of up to four dwords.
+// applies to groups that travel as one or two vectors of dwords.
 template <typename T, int N, bool NT = false>
 __device__ __forceinline__ Group<T, N> load_group(const T *p) {
     typedef Group<T, N> G;
-    if constexpr (G::kWords >= 1 && G::kWords <= 4) {
-        typedef typename WordVec<G::kWords>::type vec_t;
+    constexpr int W = G::kWords;
+    if constexpr (W >= 1 && W <= 4) {
+        typedef typename WordVec<W>::type vec_t;
         G g;
         if constexpr (NT) g.w.v = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p));
         else g.w.v = *reinterpret_cast<const vec_t *>(p);
+        return g;
+    } else if constexpr (W == 6 || W == 8) {
+        typedef typename WordVec<W / 2>::type vec_t;
+        const char *q = reinterpret_cast<const char *>(p);
+        G g;
+        if constexpr (NT) {
+            g.w.lo = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(q));
+            g.w.hi = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(q + 2 * W));
+        } else {
+            g.w.lo = *reinterpret_cast<const vec_t *>(q);
+            g.w.hi = *reinterpret_cast<const vec_t *>(q + 2 * W);
+        }
         return g;
     } else {
         return *reinterpret_cast<const G *>(p);
@@ -152,11 +169,22 @@ __device__ __forceinline__ Group<T, N> load_group(const T *p) {
 template <typename T, int N, bool NT = false>
 __device__ __forceinline__ void store_group(T *p, const float (&v)[N]) {
     typedef Group<T, N> G;
+    constexpr int W = G::kWords;
     const G g = G::make(v);
-    if constexpr (G::kWords >= 1 && G::kWords <= 4) {
-        typedef typename WordVec<G::kWords>::type vec_t;
+    if constexpr (W >= 1 && W <= 4) {
+        typedef typename WordVec<W>::type vec_t;
         if constexpr (NT) __builtin_nontemporal_store(g.w.v, reinterpret_cast<vec_t *>(p));
         else *reinterpret_cast<vec_t *>(p) = g.w.v;
+    } else if constexpr (W == 6 || W == 8) {
+        typedef typename WordVec<W / 2>::type vec_t;
+        char *q = reinterpret_cast<char *>(p);
+        if constexpr (NT) {
+            __builtin_nontemporal_store(g.w.lo, reinterpret_cast<vec_t *>(q));
+            __builtin_nontemporal_store(g.w.hi, reinterpret_cast<vec_t *>(q + 2 * W));
+        } else {
+            *reinterpret_cast<vec_t *>(q) = g.w.lo;
+            *reinterpret_cast<vec_t *>(q + 2 * W) = g.w.hi;
+        }
     } else {
         *reinterpret_cast<G *>(p) = g;
     }
