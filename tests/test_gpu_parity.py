@@ -124,6 +124,16 @@ def test_checkpointed_state(cfg, dt):
     check_against_oracle(Case(seed=24, **cfg), dt, checkpointed=True)
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("checkpointed", [False, True])
+def test_two_columns_per_lane_without_wave_uniformity(dt, checkpointed):
+    # 16-bit streams, >= 65 536 lanes at two columns per lane, d not a multiple of 128: the
+    # two-column kernels with per-lane direction / row arithmetic
+    c = Case(L=21, B=70, d=992, dirs=2, seed=25, pad="right", scale=1.7, mask_c=True)
+    assert c.B * c.Dp // 2 >= 65536 and c.d % 128 != 0
+    check_against_oracle(c, dt, checkpointed=checkpointed)
+
+
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 def test_inference_variant_without_state_store(dt):
     check_against_oracle(Case(L=40, B=4, d=128, dirs=2, seed=23, pad="right", scale=1.7), dt, keep_c=False)
