@@ -95,7 +95,12 @@ def main():
 
     import torch
     from sru_amd import _lib
-    from tests.abi import TORCH_DT, CODE, p
+
+    TORCH_DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+    CODE = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}
+
+    def p(t):   # device pointer for the C ABI
+        return None if t is None else ctypes.c_void_p(t.data_ptr())
 
     name, L, B, d, dirs, k, fwd_only, padded = WORKLOADS[args.workload]
     name += " " + args.dtype

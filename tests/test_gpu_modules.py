@@ -175,3 +175,29 @@ def test_autocast_bf16_stack_close_to_fp32():
         h16, _ = model(x)
     assert h16.dtype == torch.bfloat16
     assert float((h16.float() - h32).abs().max()) <= 2e-2 * max(1.0, float(h32.abs().max()))
+
+
+@pytest.mark.parametrize("amp_dtype", [None, torch.bfloat16, torch.float16])
+def test_training_steps_with_and_without_autocast(amp_dtype):
+    # test/test_amp.py:43-81 runs Adam steps of one SRUCell(304, 304) on a (304, 200, 304) input
+    # with and without autocast and asserts nothing; here a shorter sequence, and the loss must
+    # stay finite and go down
+    torch.manual_seed(0)
+    cell = SRUCell(304, 304, dropout=0.1, rescale=True).to(DEV)
+    opt = torch.optim.Adam(cell.parameters(), lr=3e-3)
+    x = torch.randn(48, 200, 304, device=DEV)
+    target = torch.randn(48, 200, 304, device=DEV)
+    losses = []
+    for _ in range(6):
+        opt.zero_grad()
+        if amp_dtype is None:
+            h, _ = cell(x)
+        else:
+            with torch.autocast("cuda", dtype=amp_dtype):
+                h, _ = cell(x)
+            assert h.dtype == amp_dtype
+        loss = (h.float() - target).pow(2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(np.isfinite(losses)) and losses[-1] < losses[0]
