@@ -33,6 +33,7 @@ WORKLOADS = {
     # one layer, kept for side measurements (--workload).
     "headline": ("bi-SRU d=1024 L=256 B=64 k=3", 256, 64, 1024, 2, 3, False, False),
     "headline-k4": ("bi-SRU d=1024 L=256 B=64 k=4", 256, 64, 1024, 2, 4, False, False),
+    "config1": ("uni-SRU d=128 L=20 B=32 k=3 forward only (README example)", 20, 32, 128, 1, 3, True, False),
     "config2": ("bi-SRU d=512 L=128 B=32 k=3, right-padded lengths in [32,128]", 128, 32, 512, 2, 3, False, True),
     "config4": ("uni-SRU d=2048 L=512 B=16 k=3", 512, 16, 2048, 1, 3, False, False),
     "config5": ("bi-SRU d=256 L=4096 B=256 k=3 forward only, lengths in [1024,4096]", 4096, 256, 256, 2, 3, True, True),
@@ -218,7 +219,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": name, "length": L, "batch": B, "hidden_per_direction": d,
-                   "directions": dirs, "k": k, "pass": "forward+backward, one layer",
+                   "directions": dirs, "k": k, "pass": "forward only, one layer" if fwd_only else "forward+backward, one layer",
                    "state_between_passes": "float checkpoints every 8 steps" if ckpt else "every step",
                    "buffer_sets": args.sets},
         "roofline": {"bound": "hbm", "kernel": ("backward_scan_ckpt" if ckpt else "backward_scan") + " (+ reduce_partials)",
