@@ -67,10 +67,82 @@ def cpu_baseline(L, B, d, dirs, k, budget_s=12.0):
         spent += time.perf_counter() - t0
         reps += 1
     tokens = L * Bc * reps
-    return {"value": tokens / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
-            "sample": f"{reps} x (forward+backward) of the same layer at batch {Bc} of {B} "
-                      f"(L={L}, D'={Dp}, k={k}, float32 serial C loop), {spent:.1f} s",
-            "host_cores": os.cpu_count()}
+    out = {"value": tokens / spent, "unit": "tokens/s", "cores": 1, "kind": "port",
+           "sample": f"{reps} x (forward+backward) of the same layer at batch {Bc} of {B} "
+                     f"(L={L}, D'={Dp}, k={k}, float32 serial C loop), {spent:.1f} s",
+           "host_cores": os.cpu_count()}
+    # Beside it, where the build made it: the reference's own CPU routine compiled from its
+    # source file (forward only, it has no backward), on the same arrays, one thread.
+    ref_so = os.path.join(ROOT, "oracle", "_ref", "libsru_cpu_ref.so")
+    if os.path.exists(ref_so):
+        try:
+            import torch
+            torch.ops.load_library(ref_so)
+            fn = torch.ops.sru_cpu.cpu_bi_forward if dirs == 2 else torch.ops.sru_cpu.cpu_forward
+            tU, tx, twc, tb, tc0 = (torch.from_numpy(a) for a in (U, x, wc, bias, c0))
+            threads = torch.get_num_threads()
+            torch.set_num_threads(1)
+            reps, spent = 0, 0.0
+            while reps < 1 or spent < budget_s / 3:
+                t0 = time.perf_counter()
+                fn(tU, tx, twc, tb, tc0, None, L, Bc, d, k, 0, True, 3 ** 0.5, False)
+                spent += time.perf_counter() - t0
+                reps += 1
+            torch.set_num_threads(threads)
+            out["reference_forward_only"] = {
+                "value": L * Bc * reps / spent, "unit": "tokens/s", "cores": 1, "kind": "reference",
+                "sample": f"{reps} x forward of the same layer (sru/csrc/sru_cpu_impl.cpp compiled "
+                          f"as oracle/_ref), {spent:.1f} s"}
+        except Exception as e:   # a baseline that cannot load is reported, never fatal
+            out["reference_forward_only"] = {"error": repr(e)[:200]}
+    return out
+
+
+STACKS = {
+    # key: (name, constructor arguments of sru_amd.SRU, L, B, input size, autocast dtype or None)
+    "stack3": ("4-layer bi-SRU d=1024 L=256 B=64 layer_norm rescale, module level",
+               dict(input_size=1024, hidden_size=1024, num_layers=4, bidirectional=True, layer_norm=True,
+                    rescale=True), 256, 64, 1024),
+    "stack4": ("10-layer uni-SRU hidden=2048 projection=512 L=512 B=16 dropout=0.1, module level",
+               dict(input_size=2048, hidden_size=2048, num_layers=10, projection_size=512, dropout=0.1),
+               512, 16, 2048),
+}
+
+
+def run_stack(args):
+    """Side measurement: the whole layer stack (GEMM, recurrence, layer norm, autograd) through
+    sru_amd.SRU, forward + backward per step. Not the headline metric: it shows what share of a
+    training step the recurrence kernels are and what the Python layer adds around them."""
+    import torch
+    import sru_amd
+    name, kw, L, B, n_in = STACKS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    model = sru_amd.SRU(**kw).to(dev)
+    amp = {"f32": None, "bf16": torch.bfloat16, "f16": torch.float16}[args.dtype]
+    x = torch.randn(L, B, n_in, device=dev)
+    probe = torch.randn(L, B, model.output_size, device=dev)
+
+    def step():
+        with torch.autocast("cuda", dtype=amp, enabled=amp is not None):
+            h, _ = model(x)
+        (h.float() * probe).sum().backward()
+        model.zero_grad(set_to_none=True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    print(json.dumps({
+        "metric": "module-level training step (side measurement)", "value": L * B / (ms_step * 1e-3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype if amp is None else args.dtype + " autocast", "data": "synthetic",
+        "config": {"workload": name, "length": L, "batch": B, "layers": kw["num_layers"]}}), flush=True)
 
 
 def main():
@@ -80,7 +152,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--dtype", default="f32", choices=sorted(DT_BYTES))
     ap.add_argument("--sets", type=int, default=4, help="rotating buffer sets")
-    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + sorted(STACKS))
     ap.add_argument("--full-state", action="store_true",
                     help="keep the state after every step between forward and backward, as the "
                          "reference does, instead of float checkpoints every 8 steps (the path "
@@ -93,6 +165,8 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the recurrence on ONE GPU only "
                  "(columns are independent; no multi-GPU path exists): run with --gpus 1")
+    if args.workload in STACKS:
+        return run_stack(args)
 
     import torch
     from sru_amd import _lib

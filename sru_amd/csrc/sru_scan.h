@@ -252,9 +252,11 @@ struct Stream {
 #pragma unroll
             for (int i = 0; i < N; ++i) {
                 both[i] = v[i];
-                // quad_perm [1,0,3,2]: the value of the neighbouring lane of the pair
+                // quad_perm [1,0,3,2]: the value of the neighbouring lane of the pair (every lane
+                // of a quad is a valid source, so with bound_ctrl set no previous value of the
+                // destination is needed and none has to be materialised)
                 both[N + i] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-                    0, __builtin_bit_cast(int, v[i]), 0xB1, 0xf, 0xf, false));
+                    0, __builtin_bit_cast(int, v[i]), 0xB1, 0xf, 0xf, true));
             }
             if (q == 0) store_group<T, kElems, NT>(row + (int32_t)lane * N, both);
         } else {
