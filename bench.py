@@ -32,6 +32,7 @@ WORKLOADS = {
     # metric is quoted on; the others are the reference's remaining GPU configurations at
     # one layer, kept for side measurements (--workload).
     "headline": ("bi-SRU d=1024 L=256 B=64 k=3", 256, 64, 1024, 2, 3, False, False),
+    "headline-uni": ("uni-SRU d=2048 L=256 B=64 k=3 (the headline's columns in one direction)", 256, 64, 2048, 1, 3, False, False),
     "headline-k4": ("bi-SRU d=1024 L=256 B=64 k=4", 256, 64, 1024, 2, 4, False, False),
     "config1": ("uni-SRU d=128 L=20 B=32 k=3 forward only (README example)", 20, 32, 128, 1, 3, True, False),
     "config2": ("bi-SRU d=512 L=128 B=32 k=3, right-padded lengths in [32,128]", 128, 32, 512, 2, 3, False, True),
