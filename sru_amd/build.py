@@ -11,6 +11,7 @@ SOURCES = [os.path.join(HERE, "csrc", n)
            for n in ("sru_amd.hip", "scan_f32.hip", "scan_f16.hip", "scan_bf16.hip")]
 OUTPUT = os.path.join(HERE, "libsru_amd.so")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
+SERVE_FORWARD = os.path.join(HERE, "serve_forward")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -88,7 +89,27 @@ def build(verbose=True, output=OUTPUT, defines=()):
         print(f"{len(usage)} kernels, largest scratch {max([v[1] for v in usage.values()] or [0])} bytes/lane, "
               f"largest VGPR count {max([v[0] or 0 for v in usage.values()] or [0])}", flush=True)
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", output], verbose)
+    if output == OUTPUT:
+        build_serve_forward(verbose)
     return output
+
+
+def build_serve_forward(verbose=True):
+    """Compiles csrc/serve_forward.cpp, a caller of the C ABI without Python or torch, with the
+    host compiler against the library just built (found at run time next to the program)."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-D__HIP_PLATFORM_AMD__",
+           "-I" + os.path.join(rocm, "include"), "-I" + os.path.join(ROOT, "include"),
+           os.path.join(HERE, "csrc", "serve_forward.cpp"), "-L" + HERE, "-lsru_amd",
+           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath,$ORIGIN",
+           "-Wl,-rpath," + os.path.join(rocm, "lib"), "-o", SERVE_FORWARD]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode:
+        print(proc.stdout, flush=True)
+        raise RuntimeError("host compiler failed: " + " ".join(cmd))
+    return SERVE_FORWARD
 
 
 if __name__ == "__main__":
