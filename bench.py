@@ -158,6 +158,9 @@ def main():
                     help="keep the state after every step between forward and backward, as the "
                          "reference does, instead of float checkpoints every 8 steps (the path "
                          "the autograd Function of this package takes)")
+    ap.add_argument("--tanh", action="store_true",
+                    help="side measurement of the general kernels: activation_type = tanh "
+                         "(the state after every step is kept, as those kernels need)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "
@@ -186,8 +189,10 @@ def main():
     tdt = TORCH_DT[args.dtype]
     es = DT_BYTES[args.dtype]
     lib = _lib.load()
-    ckpt = not args.full_state and not fwd_only
-    shape = _lib.Shape(L, B, d, dirs, k, 0, 1 if k == 3 else 2, 0, CODE[args.dtype],
+    ckpt = not args.full_state and not fwd_only and not args.tanh
+    if args.tanh:
+        name += " tanh"
+    shape = _lib.Shape(L, B, d, dirs, k, 1 if args.tanh else 0, 1 if k == 3 else 2, 0, CODE[args.dtype],
                        _lib.STATE_INTERVAL if ckpt else 1)
     state_rows = lib.sru_amd_state_bytes(ctypes.byref(shape)) // (B * Dp * (4 if ckpt else DT_BYTES[args.dtype]))
 
