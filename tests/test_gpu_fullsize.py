@@ -210,3 +210,27 @@ def test_offsets_beyond_32_bits_long_sequence_k4():
     h_small, cl_small = run(U[:, rows].contiguous(), c0[rows].contiguous(), pad[:, rows], 2)
     assert torch.equal(h_big[:, rows], h_small) and torch.equal(cl_big[rows], cl_small)
     assert float(h_big[pad].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("checkpointed", [False, True], ids=["state_every_step", "state_checkpoints"])
+@pytest.mark.parametrize("k", [3, 4])
+def test_long_sequence_training_against_float64_oracle(checkpointed, k):
+    """2048 steps (256 checkpoint chunks, plus a ragged tail of 5): errors of the recomputed
+    states must not build up along the walk. Same per-cell bounds as at the headline shape."""
+    c = Case(L=2053, B=3, d=96, dirs=2, k=k, seed=61, scale=1.7 if k == 3 else None, pad="right",
+             mask_c=True).f32()
+    dp = DeviceProblem(c, checkpointed=checkpointed)
+    h, cs, cl = dp.forward()
+    h_ref, c_ref, cl_ref = so.forward(*c.fwd_args(), **c.kw())
+    print()
+    _check_cells("h", to_np(h), h_ref)
+    _check_cells("c_last", to_np(cl), cl_ref)
+    gu, gx, gwc, gb, gi = dp.backward()
+    c_used = c_ref if checkpointed else to_np(cs)
+    g_ref = so.backward(*c.fwd_args(), c_used, c.gh, c.gl, **c.kw())
+    _check_cells("grad_u", to_np(gu), g_ref[0])
+    if k == 3:
+        _check_cells("grad_x", to_np(gx), g_ref[1])
+    _check_cells("grad_init", to_np(gi), g_ref[4])
+    assert _maxerr(to_np(gwc), g_ref[2]) <= 1e-5 * max(1.0, np.abs(g_ref[2]).max())
+    assert _maxerr(to_np(gb), g_ref[3]) <= 1e-5 * max(1.0, np.abs(g_ref[3]).max())
