@@ -108,3 +108,13 @@ def test_function_refuses_cpu_tensors():
     with pytest.raises(RuntimeError):
         ElementwiseRecurrence.apply(torch.randn(L, B, 3 * d), torch.randn(L, B, d), torch.randn(2 * d),
                                     torch.randn(2 * d), torch.zeros(B, d), 0, d, False, True, None)
+
+
+def test_plain_c_caller_is_built_and_links_against_the_library():
+    """sru_amd/serve_forward (no Python, no torch) starts, i.e. finds libsru_amd.so and the HIP
+    runtime next to it, and refuses a wrong argument list before it touches any device."""
+    import subprocess
+    program = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "sru_amd", "serve_forward")
+    assert os.path.exists(program), "run python -m sru_amd.build"
+    proc = subprocess.run([program], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=60)
+    assert proc.returncode == 64 and "usage:" in proc.stderr
