@@ -101,6 +101,8 @@ def cpu_baseline(L, B, d, dirs, k, budget_s=12.0):
 
 STACKS = {
     # key: (name, constructor arguments of sru_amd.SRU, L, B, input size, autocast dtype or None)
+    "stack1": ("README example: 2-layer uni-SRU d=128 L=20 B=32 highway_bias=-2, forward only, module level",
+               dict(input_size=128, hidden_size=128, num_layers=2, highway_bias=-2.0), 20, 32, 128),
     "stack3": ("4-layer bi-SRU d=1024 L=256 B=64 layer_norm rescale, module level",
                dict(input_size=1024, hidden_size=1024, num_layers=4, bidirectional=True, layer_norm=True,
                     rescale=True), 256, 64, 1024),
@@ -124,11 +126,31 @@ def run_stack(args):
     x = torch.randn(L, B, n_in, device=dev)
     probe = torch.randn(L, B, model.output_size, device=dev)
 
+    forward_only = args.workload == "stack1"
+
     def step():
+        if forward_only:
+            with torch.no_grad(), torch.autocast("cuda", dtype=amp, enabled=amp is not None):
+                return model(x)
         with torch.autocast("cuda", dtype=amp, enabled=amp is not None):
             h, _ = model(x)
         (h.float() * probe).sum().backward()
         model.zero_grad(set_to_none=True)
+
+    if args.graph:      # record the forward once, replay it per step (launch-bound shapes)
+        if not forward_only:
+            sys.exit("bench.py: --graph records the forward-only stack (stack1)")
+        model.eval()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        step = graph.replay
 
     for _ in range(args.warmup):
         step()
@@ -139,11 +161,13 @@ def run_stack(args):
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     print(json.dumps({
-        "metric": "module-level training step (side measurement)", "value": L * B / (ms_step * 1e-3),
+        "metric": "module-level step (side measurement)", "value": L * B / (ms_step * 1e-3),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype if amp is None else args.dtype + " autocast", "data": "synthetic",
-        "config": {"workload": name, "length": L, "batch": B, "layers": kw["num_layers"]}}), flush=True)
+        "config": {"workload": name, "length": L, "batch": B, "layers": kw["num_layers"],
+                   "pass": "forward only" if forward_only else "forward+backward",
+                   "replayed_from_graph": bool(args.graph)}}), flush=True)
 
 
 def main():
@@ -161,6 +185,8 @@ def main():
     ap.add_argument("--tanh", action="store_true",
                     help="side measurement of the general kernels: activation_type = tanh "
                          "(the state after every step is kept, as those kernels need)")
+    ap.add_argument("--graph", action="store_true",
+                    help="with --workload stack1: record the forward into a HIP graph and time replays")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "

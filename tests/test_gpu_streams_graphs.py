@@ -81,3 +81,32 @@ def test_autograd_function_on_second_device_stream_and_noncontiguous_inputs():
         h, last = ElementwiseRecurrence.apply(u_view, x_off, wc, bias, c0, 0, c.d, True, True, sx)
     side.synchronize()
     assert torch.equal(h, h_ref) and torch.equal(last, last_ref)
+
+
+def test_module_forward_replays_from_a_graph():
+    """The README-example stack (2 layers, d=128, L=20, B=32) is launch-bound; the whole
+    forward (GEMMs + recurrence) can be recorded once and replayed. Every replay is checked
+    against the eager result for the input it is given."""
+    import sru_amd
+    torch.manual_seed(5)
+    model = sru_amd.SRU(128, 128, num_layers=2, highway_bias=-2.0).cuda().eval()
+    static_x = torch.randn(20, 32, 128, device="cuda")
+    with torch.no_grad():
+        side = torch.cuda.Stream()          # warm-up on a side stream, as torch asks before a capture
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                model(static_x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_h, static_c = model(static_x)
+        for replay in range(3):
+            x = torch.randn(20, 32, 128, device="cuda")
+            h_eager, c_eager = model(x)          # eager work and a sync between replays
+            torch.cuda.synchronize()
+            static_x.copy_(x)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_h, h_eager), replay
+            assert torch.equal(static_c, c_eager), replay
