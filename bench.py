@@ -103,6 +103,8 @@ STACKS = {
     # key: (name, constructor arguments of sru_amd.SRU, L, B, input size, autocast dtype or None)
     "stack1": ("README example: 2-layer uni-SRU d=128 L=20 B=32 highway_bias=-2, forward only, module level",
                dict(input_size=128, hidden_size=128, num_layers=2, highway_bias=-2.0), 20, 32, 128),
+    "stack2": ("4-layer bi-SRU d=512 L=128 B=32, right-padded lengths in [32,128], module level",
+               dict(input_size=512, hidden_size=512, num_layers=4, bidirectional=True), 128, 32, 512),
     "stack3": ("4-layer bi-SRU d=1024 L=256 B=64 layer_norm rescale, module level",
                dict(input_size=1024, hidden_size=1024, num_layers=4, bidirectional=True, layer_norm=True,
                     rescale=True), 256, 64, 1024),
@@ -127,13 +129,17 @@ def run_stack(args):
     probe = torch.randn(L, B, model.output_size, device=dev)
 
     forward_only = args.workload == "stack1"
+    mask_pad = None
+    if args.workload == "stack2":
+        lens = torch.randint(32, L + 1, (B,), device=dev)
+        mask_pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :])
 
     def step():
         if forward_only:
             with torch.no_grad(), torch.autocast("cuda", dtype=amp, enabled=amp is not None):
                 return model(x)
         with torch.autocast("cuda", dtype=amp, enabled=amp is not None):
-            h, _ = model(x)
+            h, _ = model(x, mask_pad=mask_pad)
         (h.float() * probe).sum().backward()
         model.zero_grad(set_to_none=True)
 
