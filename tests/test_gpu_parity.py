@@ -12,6 +12,8 @@ Tolerances (the bar the build is held to):
                     float64 oracle fed the same rounded inputs.
 Outputs are pre-filled with NaN: a cell the kernels do not write fails the comparison.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -183,3 +185,35 @@ def test_backward_is_bit_reproducible():
     for _ in range(3):
         again = a.backward()
         assert all(torch.equal(p, q) for p, q in zip(first, again))
+
+
+def _random_cases(n, seed):
+    """Seeded draw over everything the boundary accepts: sizes around the wavefront, pair and
+    chunk boundaries, both directions, every flag combination the shape check allows."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        k = int(rng.choice([3, 4]))
+        skip = bool(rng.random() < 0.85)
+        cfg = dict(L=int(rng.choice([1, 2, 7, 8, 9, 15, 16, 17, 23, 24, 31, 40])),
+                   B=int(rng.integers(1, 6)),
+                   d=int(rng.choice([1, 2, 3, 31, 32, 33, 63, 64, 65, 96, 127, 128, 130, 192])),
+                   dirs=int(rng.choice([1, 2])), k=k, skip=skip,
+                   act=int(rng.random() < 0.2), custom=bool(rng.random() < 0.15),
+                   pad=[None, "right", "random"][int(rng.integers(0, 3))],
+                   mask_c=bool(rng.random() < 0.4),
+                   scale=float(rng.choice([1.0, 0.6, 1.7])) if (k == 3 and skip) else None,
+                   zero_c0=bool(rng.random() < 0.3))
+        dt = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+        out.append((cfg, dt, bool(rng.random() < 0.5), 1000 + i))
+    return out
+
+
+# SRU_AMD_RANDOM_CASES / SRU_AMD_RANDOM_SEED widen or move the draw for a one-off sweep
+@pytest.mark.parametrize("cfg,dt,checkpointed,seed",
+                         _random_cases(int(os.environ.get("SRU_AMD_RANDOM_CASES", "60")),
+                                       int(os.environ.get("SRU_AMD_RANDOM_SEED", "2024"))),
+                         ids=lambda v: _ids(v) if isinstance(v, dict) else str(v))
+def test_random_draws_over_shapes_and_flags(cfg, dt, checkpointed, seed):
+    fast = cfg["skip"] and not cfg["act"] and not cfg["custom"]
+    check_against_oracle(Case(seed=seed, **cfg), dt, checkpointed=checkpointed and fast)
