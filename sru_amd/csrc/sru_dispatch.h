@@ -182,13 +182,13 @@ void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) 
         if (s.k == 3) pick_forward<T, 3, 1>(s, p, st);
         else pick_forward<T, 4, 2>(s, p, st);
     } else if (s.k == 3 && s.skip_type == 1) {
-        hipLaunchKernelGGL((forward_scan<T, 3, 1, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((forward_scan<T, 3, 1, kGeneral | kFwdNt, 1, P>), grid, block, 0, st, p);
     } else if (s.k == 3) {
-        hipLaunchKernelGGL((forward_scan<T, 3, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((forward_scan<T, 3, 0, kGeneral | kFwdNt, 1, P>), grid, block, 0, st, p);
     } else if (s.skip_type == 2) {
-        hipLaunchKernelGGL((forward_scan<T, 4, 2, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((forward_scan<T, 4, 2, kGeneral | kFwdNt, 1, P>), grid, block, 0, st, p);
     } else {
-        hipLaunchKernelGGL((forward_scan<T, 4, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((forward_scan<T, 4, 0, kGeneral | kFwdNt, 1, P>), grid, block, 0, st, p);
     }
 }
 
@@ -201,13 +201,13 @@ void launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st)
         if (s.k == 3) pick_backward<T, 3, 1>(s, p, st);
         else pick_backward<T, 4, 2>(s, p, st);
     } else if (s.k == 3 && s.skip_type == 1) {
-        hipLaunchKernelGGL((backward_scan<T, 3, 1, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((backward_scan<T, 3, 1, kGeneral | kBwdNt, 1, P>), grid, block, 0, st, p);
     } else if (s.k == 3) {
-        hipLaunchKernelGGL((backward_scan<T, 3, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((backward_scan<T, 3, 0, kGeneral | kBwdNt, 1, P>), grid, block, 0, st, p);
     } else if (s.skip_type == 2) {
-        hipLaunchKernelGGL((backward_scan<T, 4, 2, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((backward_scan<T, 4, 2, kGeneral | kBwdNt, 1, P>), grid, block, 0, st, p);
     } else {
-        hipLaunchKernelGGL((backward_scan<T, 4, 0, kGeneral, 1, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((backward_scan<T, 4, 0, kGeneral | kBwdNt, 1, P>), grid, block, 0, st, p);
     }
 }
 
