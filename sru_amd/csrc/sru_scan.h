@@ -480,6 +480,13 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
     constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
+    // Wave-uniform kernels with a padding mask: all lanes of a wavefront share the flags, so one
+    // load per chunk fetches them (lane l the flag of step l % TC) instead of one load per step,
+    // which leaves more of the 64 outstanding memory operations a wavefront may have to the
+    // streams: 4 % at L=4096 fp16 inference. Not with lane pairing: those shapes are short of
+    // issue slots, and reading a flag back from its lane costs one instruction more per step.
+    constexpr bool PAD_BY_LANE = HAS_PAD && UNI && !PAIR;
+    constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
@@ -522,7 +529,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     struct Chunk {
         typename SU::G u[TC];
         typename S1::G x[TC];
-        uint32_t pad[TC];
+        uint32_t pad[kPadRegs];  // padding flags of the chunk, see load_chunk
     };
 
     auto load_chunk = [&](Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
@@ -533,9 +540,12 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
                 const int64_t e = ef + (s0 + i) * es;
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
                 if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
-                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
+                if (!PAD_BY_LANE) k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
+        // one load for the whole chunk: lane l fetches the flag of step l % TC (clamped to the
+        // chunk's last valid step), compute_chunk reads step i's flag from lane i
+        if (PAD_BY_LANE) k.pad[0] = p.pad[pf + (s0 + min((int)(threadIdx.x % TC), n - 1)) * ps];
     };
 
     auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
@@ -543,7 +553,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
-                const bool padded = k.pad[i] != 0;
+                const bool padded = (PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i]) != 0;
                 float hv[COLS], cv[COLS], uu[COLS * K], xx[COLS] = {};
                 SU::unpack(k.u[i], q, uu);
                 if (SKIP == 1) S1::unpack(k.x[i], q, xx);
@@ -794,6 +804,10 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
+    // (forward_scan_chunked fetches the flags of a chunk with one load; here, where every flag
+    // is needed twice, that measured 0-3 % slower, so the flags stay one load per step)
+    constexpr bool PAD_BY_LANE = false;
+    constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
@@ -841,7 +855,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         typename SU::G u[TC];
         typename S1::G x[TC];
         typename S1::G gh[TC];
-        uint32_t pad[TC];
+        uint32_t pad[kPadRegs];  // padding flags of the chunk, see load_chunk
         float cstart[COLS];  // state before the chunk's first step
     };
 
@@ -855,9 +869,10 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
                 if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
                 k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
-                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
+                if (!PAD_BY_LANE) k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
+        if (PAD_BY_LANE) k.pad[0] = p.pad[pf + (s0 + min((int)(threadIdx.x % TC), n - 1)) * ps];  // see forward_scan_chunked
 #pragma unroll
         for (int c = 0; c < COLS; ++c)
             k.cstart[c] = (ch == 0) ? c_init[c] : p.ckpt[(ch - 1) * p.ncols + col + c];
@@ -873,7 +888,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
-                const bool padded = k.pad[i] != 0;
+                const bool padded = (PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i]) != 0;
                 float uu[COLS * K];
                 SU::unpack(k.u[i], q, uu);
 #pragma unroll
@@ -891,7 +906,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
 #pragma unroll
         for (int i = TC - 1; i >= 0; --i) {
             if (i < n) {
-                const bool padded = k.pad[i] != 0;
+                const bool padded = (PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i]) != 0;
                 float gu[COLS * K], gx[COLS], xx[COLS] = {}, ghs[COLS];
                 if (SKIP == 1) S1::unpack(k.x[i], q, xx);
                 S1::unpack(k.gh[i], q, ghs);
