@@ -110,3 +110,39 @@ def test_module_forward_replays_from_a_graph():
             torch.cuda.synchronize()
             assert torch.equal(static_h, h_eager), replay
             assert torch.equal(static_c, c_eager), replay
+
+
+def test_two_host_threads_on_two_streams():
+    """The library keeps no state between calls: two host threads, each with its own stream and
+    buffers, run forward + backward at the same time and get what they get alone."""
+    import threading
+    cases = [Case(L=48, B=4, d=128, dirs=2, seed=71, pad="right", scale=1.7),
+             Case(L=40, B=3, d=192, dirs=1, k=4, seed=72, mask_c=True)]
+    problems = [DeviceProblem(c, checkpointed=True) for c in cases]
+    alone = []
+    for dp in problems:
+        alone.append([t.clone() for t in dp.forward()] + [t.clone() for t in dp.backward() if t is not None])
+    torch.cuda.synchronize()
+    together = [None, None]
+    errors = []
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    out = list(problems[i].forward()) + [t for t in problems[i].backward() if t is not None]
+            stream.synchronize()
+            together[i] = out
+        except Exception as e:      # surfaced below, in the test's own thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for a, b in zip(alone, together):
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
