@@ -96,7 +96,35 @@ def cpu_baseline(L, B, d, dirs, k, budget_s=12.0):
                           f"as oracle/_ref), {spent:.1f} s"}
         except Exception as e:   # a baseline that cannot load is reported, never fatal
             out["reference_forward_only"] = {"error": repr(e)[:200]}
+    out["python_autograd_loop"] = cpu_autograd_loop()
     return out
+
+
+def cpu_autograd_loop(budget_s=3.0):
+    """The reference's other CPU path, the Python loop over time under autograd
+    (sru/ops.py:145-250), as restated in oracle/sru_torch.py: forward + backward at the small
+    shapes it is practical for (configs 1 and 2, one layer), float32, torch's default threads."""
+    import torch
+    from oracle import sru_torch as st
+    res = {"unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port"}
+    for key, (L, B, d, bi) in {"config1": (20, 32, 128, False), "config2": (128, 32, 512, True)}.items():
+        g = torch.Generator().manual_seed(0)
+        Dp = d * (2 if bi else 1)
+        u = torch.randn(L, B, Dp * 3, generator=g, requires_grad=True)
+        x = torch.randn(L, B, Dp, generator=g, requires_grad=True)
+        wc = torch.randn(2 * Dp, generator=g, requires_grad=True)
+        bias = torch.zeros(2 * Dp, requires_grad=True)
+        c0 = torch.zeros(B, Dp, requires_grad=True)
+        probe = torch.randn(L, B, Dp, generator=g)
+        reps, spent = 0, 0.0
+        while reps < 1 or spent < budget_s:
+            t0 = time.perf_counter()
+            h, last = st.recurrence(u, x, wc, bias, c0, 0, d, bi, True, torch.tensor([3 ** 0.5]))
+            (h * probe).sum().backward()
+            spent += time.perf_counter() - t0
+            reps += 1
+        res[key] = {"value": L * B * reps / spent, "sample": f"{reps} x (forward+backward), L={L} B={B} D'={Dp}, {spent:.1f} s"}
+    return res
 
 
 STACKS = {
