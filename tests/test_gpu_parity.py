@@ -217,3 +217,19 @@ def _random_cases(n, seed):
 def test_random_draws_over_shapes_and_flags(cfg, dt, checkpointed, seed):
     fast = cfg["skip"] and not cfg["act"] and not cfg["custom"]
     check_against_oracle(Case(seed=seed, **cfg), dt, checkpointed=checkpointed and fast)
+
+
+@pytest.mark.parametrize("checkpointed", [False, True])
+@pytest.mark.parametrize("act", [0, 1])
+def test_saturated_gates_stay_finite(checkpointed, act):
+    """Gate inputs of magnitude up to 1e4: the sigmoids are exactly 0 or 1 in float, exp2
+    overflows to infinity inside them, and neither pass may turn that into NaN."""
+    if checkpointed and act:
+        pytest.skip("checkpointed state exists for the fast kernels only")
+    c = Case(L=24, B=3, d=64, dirs=2, seed=88, scale=1.3, pad="right", act=act)
+    rng = np.random.default_rng(5)
+    big = rng.choice([-1e4, -100.0, 100.0, 1e4], size=c.U.shape)
+    hit = rng.random(c.U.shape) < 0.3
+    hit.reshape(c.L, c.B, c.Dp, c.k)[..., 0] = False      # gate streams only; u0 stays moderate
+    c.U = np.where(hit, big, c.U)
+    check_against_oracle(c.f32(), "f32", checkpointed=checkpointed)
