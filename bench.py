@@ -216,9 +216,11 @@ def main():
                     help="keep the state after every step between forward and backward, as the "
                          "reference does, instead of float checkpoints every 8 steps (the path "
                          "the autograd Function of this package takes)")
+    ap.add_argument("--no-skip", action="store_true",
+                    help="side measurement of the general kernels: no skip term (has_skip_term=False; "
+                         "the state after every step is kept, as those kernels need)")
     ap.add_argument("--tanh", action="store_true",
-                    help="side measurement of the general kernels: activation_type = tanh "
-                         "(the state after every step is kept, as those kernels need)")
+                    help="side measurement: activation_type = tanh (the reference's deprecated use_tanh)")
     ap.add_argument("--graph", action="store_true",
                     help="with --workload stack1: record the forward into a HIP graph and time replays")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -249,10 +251,14 @@ def main():
     tdt = TORCH_DT[args.dtype]
     es = DT_BYTES[args.dtype]
     lib = _lib.load()
-    ckpt = not args.full_state and not fwd_only and not args.tanh
+    ckpt = not args.full_state and not fwd_only and not args.no_skip
+    use_x = k == 3 and not args.no_skip      # the skip term is read from x
     if args.tanh:
         name += " tanh"
-    shape = _lib.Shape(L, B, d, dirs, k, 1 if args.tanh else 0, 1 if k == 3 else 2, 0, CODE[args.dtype],
+    if args.no_skip:
+        name += " no skip term"
+    shape = _lib.Shape(L, B, d, dirs, k, 1 if args.tanh else 0,
+                       0 if args.no_skip else (1 if k == 3 else 2), 0, CODE[args.dtype],
                        _lib.STATE_INTERVAL if ckpt else 1)
     state_rows = lib.sru_amd_state_bytes(ctypes.byref(shape)) // (B * Dp * (4 if ckpt else DT_BYTES[args.dtype]))
 
@@ -287,17 +293,17 @@ def main():
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
 
     def fwd(s):
-        rc = lib.sru_amd_forward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if k == 3 else None, p(wc), p(bias),
-                                 p(c0), None, p(pad), p(scale) if k == 3 else None, p(s["h"]),
+        rc = lib.sru_amd_forward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if use_x else None, p(wc), p(bias),
+                                 p(c0), None, p(pad), p(scale) if use_x else None, p(s["h"]),
                                  None if fwd_only else p(s["c"]), p(c_last), stream)
         assert rc == 0, _lib.status_string(rc)
 
     def bwd(s):
         if fwd_only:
             return
-        rc = lib.sru_amd_backward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if k == 3 else None, p(wc), p(bias),
-                                  p(c0), None, p(pad), p(scale) if k == 3 else None, p(s["c"]), p(s["gh"]),
-                                  p(gl), p(s["gu"]), p(s["gx"]) if k == 3 else None,
+        rc = lib.sru_amd_backward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if use_x else None, p(wc), p(bias),
+                                  p(c0), None, p(pad), p(scale) if use_x else None, p(s["c"]), p(s["gh"]),
+                                  p(gl), p(s["gu"]), p(s["gx"]) if use_x else None,
                                   p(gwc), p(gb), p(gi), p(ws), ctypes.c_size_t(ws_bytes), stream)
         assert rc == 0, _lib.status_string(rc)
 
@@ -346,8 +352,10 @@ def main():
     tfile = os.path.join(ROOT, "profiles", "traffic_bi_d1024_L256_B64_%s.json" % args.dtype)
     if args.workload == "headline" and ckpt and os.path.exists(tfile):
         traffic = json.load(open(tfile))["backward_scan"]["traffic_bytes"]
-    fwd_bytes = (5 if fwd_only else 6) * es * cells   # reads U (k) and x (k=3), writes h and (training) c
-    bwd_bytes = 10 * es * cells    # reads U (k), x (k=3), c, grad_h; writes grad_u (k), grad_x (k=3)
+    # forward reads U (k) and x (k=3 with a skip term), writes h and (training) c;
+    # backward reads U (k), x, c, grad_h and writes grad_u (k), grad_x
+    fwd_bytes = (k + (1 if use_x else 0) + (1 if fwd_only else 2)) * es * cells
+    bwd_bytes = (2 * k + (2 if use_x else 0) + 2) * es * cells
     if fwd_only:
         bwd_us = float("nan")
     bwd_gbs = bwd_bytes / (bwd_us * 1e-6) / 1e9

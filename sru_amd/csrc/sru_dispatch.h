@@ -1,9 +1,9 @@
 // Kernel selection for one stream element type T. Included by scan_<type>.hip only.
 //
 // Fast kernels exist for the two layouts the SRU layer produces with a skip term and no
-// tanh / per-step weight_c: (k=3, skip from x) and (k=4, skip from U[..., 3]); whether a
-// padding mask is given and whether c is stored are compiled in. Everything else (tanh,
-// per-step weight_c, no skip term) runs the general kernels, one column per lane.
+// per-step weight_c: (k=3, skip from x) and (k=4, skip from U[..., 3]); whether a padding
+// mask is given, whether and how c is stored and the activation are compiled in. Everything
+// else (per-step weight_c, no skip term) runs the general kernels, one column per lane.
 #pragma once
 
 #include "sru_launch.h"
@@ -87,15 +87,19 @@ bool pair_ok(const sru_amd_shape &s, std::initializer_list<const void *> wide,
 #endif
 inline bool wave_uniform(int32_t d, int cols) { return SRU_AMD_UNIFORM && d % (kBlock * cols) == 0; }
 
-template <typename T, int K, int SKIP, int COLS, int PAIR = 0, int UNI = -1>
+template <typename T, int K, int SKIP, int COLS, int PAIR = 0, int UNI = -1, int ACT = -1>
 void fast_forward(const FwdParams &p, hipStream_t st) {
+    if constexpr (ACT < 0) {   // the activation is a template bit of the fast kernels
+        if (p.act) return fast_forward<T, K, SKIP, COLS, PAIR, UNI, kTanh>(p, st);
+        return fast_forward<T, K, SKIP, COLS, PAIR, UNI, 0>(p, st);
+    }
 #if SRU_AMD_FWD_CHUNKED
     if constexpr (UNI < 0) {   // pick the scalar-addressing build of the kernel when the shape allows
-        if (wave_uniform(p.d, COLS)) return fast_forward<T, K, SKIP, COLS, PAIR, kUniform>(p, st);
-        return fast_forward<T, K, SKIP, COLS, PAIR, 0>(p, st);
+        if (wave_uniform(p.d, COLS)) return fast_forward<T, K, SKIP, COLS, PAIR, kUniform, ACT>(p, st);
+        return fast_forward<T, K, SKIP, COLS, PAIR, 0, ACT>(p, st);
     }
 #endif
-    constexpr int X = PAIR | (UNI > 0 ? UNI : 0);
+    constexpr int X = PAIR | (UNI > 0 ? UNI : 0) | (ACT > 0 ? ACT : 0);
     constexpr int P = Tune<T>::kFwdDepth;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
     // what is kept for the backward pass: nothing, the state after every step, or checkpoints
@@ -114,33 +118,38 @@ void fast_forward(const FwdParams &p, hipStream_t st) {
 #else
     static_assert(PAIR == 0, "lane pairing exists in the chunked kernels only");
     switch (mode) {
-    case 0: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kFwdNt, COLS, P>), grid, block, 0, st, p); break;
-    case kHasPad: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
-    case kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kKeepC | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
-    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kKeepC | kFwdNt, COLS, P>), grid, block, 0, st, p); break;
-    case kCkpt: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kCkpt | kFwdNt, COLS, kCkptInterval>), grid, block, 0, st, p); break;
-    default: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kCkpt | kFwdNt, COLS, kCkptInterval>), grid, block, 0, st, p); break;
+    case 0: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kFwdNt | (ACT > 0 ? ACT : 0), COLS, P>), grid, block, 0, st, p); break;
+    case kHasPad: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kFwdNt | (ACT > 0 ? ACT : 0), COLS, P>), grid, block, 0, st, p); break;
+    case kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kKeepC | kFwdNt | (ACT > 0 ? ACT : 0), COLS, P>), grid, block, 0, st, p); break;
+    case kHasPad | kKeepC: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kKeepC | kFwdNt | (ACT > 0 ? ACT : 0), COLS, P>), grid, block, 0, st, p); break;
+    case kCkpt: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kCkpt | kFwdNt | (ACT > 0 ? ACT : 0), COLS, kCkptInterval>), grid, block, 0, st, p); break;
+    default: hipLaunchKernelGGL((forward_scan<T, K, SKIP, kHasPad | kCkpt | kFwdNt | (ACT > 0 ? ACT : 0), COLS, kCkptInterval>), grid, block, 0, st, p); break;
     }
 #endif
 }
 
-template <typename T, int K, int SKIP, int COLS, int PAIR = 0>
+template <typename T, int K, int SKIP, int COLS, int PAIR = 0, int ACT = -1>
 void fast_backward(const BwdParams &p, hipStream_t st) {
+    if constexpr (ACT < 0) {
+        if (p.act) return fast_backward<T, K, SKIP, COLS, PAIR, kTanh>(p, st);
+        return fast_backward<T, K, SKIP, COLS, PAIR, 0>(p, st);
+    }
+    constexpr int A = ACT > 0 ? ACT : 0;
     constexpr int P = Tune<T>::kBwdDepth;
     constexpr int TC = kCkptInterval;
     const dim3 grid = grid_for(p.ncols, COLS), block(kBlock);
     if (p.ckpt) {
         const int mode = (p.pad ? 1 : 0) | (wave_uniform(p.d, COLS) ? 2 : 0);
         switch (mode) {
-        case 0: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); break;
-        case 1: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR, COLS, TC>), grid, block, 0, st, p); break;
-        case 2: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR | kUniform, COLS, TC>), grid, block, 0, st, p); break;
-        default: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR | kUniform, COLS, TC>), grid, block, 0, st, p); break;
+        case 0: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR | A, COLS, TC>), grid, block, 0, st, p); break;
+        case 1: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR | A, COLS, TC>), grid, block, 0, st, p); break;
+        case 2: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kBwdNt | PAIR | A | kUniform, COLS, TC>), grid, block, 0, st, p); break;
+        default: hipLaunchKernelGGL((backward_scan_ckpt<T, K, SKIP, kHasPad | kBwdNt | PAIR | A | kUniform, COLS, TC>), grid, block, 0, st, p); break;
         }
     } else if (p.pad) {
-        hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad | kBwdNt, COLS, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((backward_scan<T, K, SKIP, kHasPad | kBwdNt | A, COLS, P>), grid, block, 0, st, p);
     } else {
-        hipLaunchKernelGGL((backward_scan<T, K, SKIP, kBwdNt, COLS, P>), grid, block, 0, st, p);
+        hipLaunchKernelGGL((backward_scan<T, K, SKIP, kBwdNt | A, COLS, P>), grid, block, 0, st, p);
     }
 }
 
@@ -175,7 +184,7 @@ void pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
 // (k, skip_type) pairs that pass the shape check: (3,0) (3,1) (4,0) (4,2).
 template <typename T>
 void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
-    const bool general = s.activation_type != 0 || s.is_custom != 0 || s.skip_type == 0;
+    const bool general = s.is_custom != 0 || s.skip_type == 0;
     const dim3 grid = grid_for(p.ncols, 1), block(kBlock);
     constexpr int P = kGeneralDepth;
     if (!general) {
@@ -194,7 +203,7 @@ void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) 
 
 template <typename T>
 void launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
-    const bool general = s.activation_type != 0 || s.is_custom != 0 || s.skip_type == 0;
+    const bool general = s.is_custom != 0 || s.skip_type == 0;
     const dim3 grid = grid_for(p.ncols, 1), block(kBlock);
     constexpr int P = kGeneralDepth;
     if (!general) {

@@ -272,6 +272,13 @@ __device__ __forceinline__ float sigmoid(float v) {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
 }
 
+// tanh through the same two units: 1 - 2 / (1 + e^(2v)). Absolute error below 3e-7 over the
+// whole real line (the cancellation near 0 costs relative, not absolute, accuracy); saturates
+// cleanly to -1 and 1.
+__device__ __forceinline__ float tanh_fast(float v) {
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * v));
+}
+
 // ---------------------------------------------------------------- kernel parameters
 struct FwdParams {
     const void *u, *x, *wc;
@@ -305,9 +312,9 @@ struct BwdParams {
 // The loop body must stay one straight line of code for the compiler to keep the ring
 // in fixed registers and count outstanding loads (a uniform branch inside it makes the
 // inserted waits drain the ring at every step). The fast kernels therefore take "is
-// there a padding mask" and "is the per-step state kept" as template bits; the general
-// kernels read those and the rarely used tanh / per-step weight_c options from the
-// parameter block.
+// there a padding mask", "is the per-step state kept" and the activation as template
+// bits; the general kernels read those and the rarely used per-step weight_c option
+// from the parameter block.
 constexpr int kHasPad = 1;   // MODE bit (fast kernels): mask_pad given
 constexpr int kKeepC = 2;    // MODE bit (fast forward kernels): c is stored
 constexpr int kGeneral = 4;  // MODE bit: run-time pad / keep_c / act / custom
@@ -315,6 +322,7 @@ constexpr int kNtLoad = 8;   // MODE bit: stream loads are non-temporal
 constexpr int kNtStore = 16; // MODE bit: stream stores are non-temporal
 constexpr int kCkpt = 32;    // MODE bit (fast forward kernels): store a state checkpoint per chunk
 constexpr int kPair = 64;    // MODE bit (chunked fast kernels, 16-bit): lanes pair up for memory access
+constexpr int kTanh = 256;   // MODE bit (fast kernels): the output uses tanh(c_t) instead of c_t
 constexpr int kUniform = 128;// MODE bit (chunked fast kernels): a wavefront lies inside one direction and
                              // one batch row (d is a multiple of 64 * COLS), so the time index, the row
                              // pointers and the padding flag are scalar: no per-lane address arithmetic
@@ -344,7 +352,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     const int64_t b = col / Dp;
     const bool flip = j >= p.d;  // second direction; never true when dirs == 1 (d == D')
     const bool custom = GENERAL && p.custom;
-    const bool use_tanh = GENERAL && p.act;
+    const bool use_tanh = GENERAL ? (p.act != 0) : ((MODE & kTanh) != 0);
     const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
     const bool keep_c = GENERAL ? (p.c != nullptr) : ((MODE & kKeepC) != 0);
 
@@ -414,7 +422,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             const float g1 = sigmoid(u1 + w1 * cur[c] + b1[c]);
             const float g2 = sigmoid(u2 + w2 * cur[c] + b2[c]);
             const float cn = (cur[c] - u0) * g1 + u0;
-            const float val = use_tanh ? tanhf(cn) : cn;
+            const float val = use_tanh ? tanh_fast(cn) : cn;
             float out;
             if (SKIP != 0) {
                 const float xv = (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
@@ -480,6 +488,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
     constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
+    constexpr bool TANH = (MODE & kTanh) != 0;
     // Wave-uniform kernels with a padding mask: all lanes of a wavefront share the flags, so one
     // load per chunk fetches them (lane l the flag of step l % TC) instead of one load per step,
     // which leaves more of the 64 outstanding memory operations a wavefront may have to the
@@ -564,7 +573,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
                     const float g2 = sigmoid(uu[c * K + 2] + wc2[c] * cur[c] + b2[c]);
                     const float cn = (cur[c] - u0) * g1 + u0;
                     const float xv = (SKIP == 1) ? xx[c] * sx : uu[c * K + K - 1];
-                    const float out = (cn - xv) * m[c] * g2 + xv;
+                    const float val = TANH ? tanh_fast(cn) : cn;
+                    const float out = (val - xv) * m[c] * g2 + xv;
                     cur[c] = padded ? cur[c] : cn;
                     hv[c] = padded ? 0.0f : out;
                     cv[c] = cur[c];
@@ -633,7 +643,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
     const int64_t b = col / Dp;
     const bool flip = j >= p.d;
     const bool custom = GENERAL && p.custom;
-    const bool use_tanh = GENERAL && p.act;
+    const bool use_tanh = GENERAL ? (p.act != 0) : ((MODE & kTanh) != 0);
     const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
 
     float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
@@ -720,7 +730,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
             const float u0 = s.u.get(c * K);
             const float g1 = sigmoid(s.u.get(c * K + 1) + w1 * cp + b1[c]);
             const float g2 = sigmoid(s.u.get(c * K + 2) + w2 * cp + b2[c]);
-            const float val = use_tanh ? tanhf(cv[c]) : cv[c];
+            const float val = use_tanh ? tanh_fast(cv[c]) : cv[c];
             const float dact = use_tanh ? (1.0f - val * val) : 1.0f;
             const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
             const float gh = s.gh.get(c);
@@ -807,6 +817,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     // (forward_scan_chunked fetches the flags of a chunk with one load; here, where every flag
     // is needed twice, that measured 0-3 % slower, so the flags stay one load per step)
     constexpr bool PAD_BY_LANE = false;
+    constexpr bool TANH = (MODE & kTanh) != 0;
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
@@ -912,14 +923,16 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 S1::unpack(k.gh[i], q, ghs);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
-                    const float cp = st[i][c], val = st[i + 1][c];
+                    const float cp = st[i][c];
+                    const float val = TANH ? tanh_fast(st[i + 1][c]) : st[i + 1][c];
+                    const float dact = TANH ? (1.0f - val * val) : 1.0f;
                     const float u0 = u0s[i][c];
                     const float G1 = g1[i][c], G2 = g2[i][c];
                     const float xv = (SKIP == 1) ? xx[c] * sx : xs[i][c];
                     const float gh = ghs[c];
 
                     const float gg2 = gh * (val - xv) * m[c] * (G2 * (1.0f - G2));
-                    const float gc = gh * m[c] * G2 + cur[c];
+                    const float gc = TANH ? gh * m[c] * (G2 * dact) + cur[c] : gh * m[c] * G2 + cur[c];
                     const float gg1 = gc * (cp - u0) * (G1 * (1.0f - G1));
                     const float gskip = gh * (1.0f - G2 * m[c]);
                     const float ncur = gc * G1 + gg1 * wc1[c] + gg2 * wc2[c];

@@ -107,6 +107,8 @@ MID = [
     dict(L=64, B=8, d=256, dirs=2, pad="right", scale=1.7, mask_c=True),
     dict(L=25, B=2, d=64, dirs=2, custom=True, pad="right"),
     dict(L=25, B=2, d=64, dirs=2, act=1, k=4),
+    dict(L=19, B=3, d=128, dirs=2, act=1, pad="right", scale=1.3, mask_c=True),
+    dict(L=33, B=2, d=70, act=1, pad="random"),
     dict(L=25, B=2, d=64, skip=False, pad="random"),
 ]
 
@@ -117,7 +119,7 @@ def test_mid_shapes(cfg, dt):
     check_against_oracle(Case(seed=22, **cfg), dt)
 
 
-FAST = [g for g in GRID + MID if not g.get("custom") and not g.get("act") and g.get("skip", True)]
+FAST = [g for g in GRID + MID if not g.get("custom") and g.get("skip", True)]
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
@@ -215,7 +217,7 @@ def _random_cases(n, seed):
                                        int(os.environ.get("SRU_AMD_RANDOM_SEED", "2024"))),
                          ids=lambda v: _ids(v) if isinstance(v, dict) else str(v))
 def test_random_draws_over_shapes_and_flags(cfg, dt, checkpointed, seed):
-    fast = cfg["skip"] and not cfg["act"] and not cfg["custom"]
+    fast = cfg["skip"] and not cfg["custom"]
     check_against_oracle(Case(seed=seed, **cfg), dt, checkpointed=checkpointed and fast)
 
 
@@ -224,8 +226,6 @@ def test_random_draws_over_shapes_and_flags(cfg, dt, checkpointed, seed):
 def test_saturated_gates_stay_finite(checkpointed, act):
     """Gate inputs of magnitude up to 1e4: the sigmoids are exactly 0 or 1 in float, exp2
     overflows to infinity inside them, and neither pass may turn that into NaN."""
-    if checkpointed and act:
-        pytest.skip("checkpointed state exists for the fast kernels only")
     c = Case(L=24, B=3, d=64, dirs=2, seed=88, scale=1.3, pad="right", act=act)
     rng = np.random.default_rng(5)
     big = rng.choice([-1e4, -100.0, 100.0, 1e4], size=c.U.shape)
