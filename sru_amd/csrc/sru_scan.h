@@ -290,7 +290,7 @@ struct FwdParams {
     float *ckpt;          // (L / kCkptInterval, B, D') float state checkpoints, or nullptr
     int64_t L, B, ncols;  // ncols = B * D'
     int32_t d, Dp;        // hidden per direction, D' = dirs * d
-    int32_t act, custom;  // only read by the general kernels
+    int32_t act, custom;  // act: host-side kernel selection and the general kernels; custom: general kernels
 };
 
 struct BwdParams {
