@@ -8,7 +8,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SOURCES = [os.path.join(HERE, "csrc", n)
-           for n in ("sru_amd.hip", "scan_f32.hip", "scan_f16.hip", "scan_bf16.hip")]
+           for n in ("sru_amd.hip", "scan_f32_fwd.hip", "scan_f32_bwd.hip", "scan_f16_fwd.hip",
+                     "scan_f16_bwd.hip", "scan_bf16_fwd.hip", "scan_bf16_bwd.hip")]
 OUTPUT = os.path.join(HERE, "libsru_amd.so")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 SERVE_FORWARD = os.path.join(HERE, "serve_forward")
@@ -76,7 +77,7 @@ def build(verbose=True, output=OUTPUT, defines=()):
     jobs = [[hipcc] + HIPCC_FLAGS + extra + ["-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
             for src, obj in zip(SOURCES, objs)]
     usage = {}
-    with ThreadPoolExecutor(max_workers=4) as pool:
+    with ThreadPoolExecutor(max_workers=len(jobs)) as pool:
         for part in pool.map(lambda cmd: _run(cmd, verbose), jobs):
             usage.update(part)
     with open(os.path.join(obj_dir, "resource_usage.json"), "w") as f:

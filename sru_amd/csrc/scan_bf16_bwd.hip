@@ -1,7 +1,6 @@
-// Scan kernels and their launchers for bf16_bits streams.
+// Backward scan kernels and their launcher for bf16_bits streams.
 #include "sru_dispatch.h"
 
 namespace sru_amd {
-template void launch_forward<bf16_bits>(const sru_amd_shape &, const FwdParams &, hipStream_t);
 template void launch_backward<bf16_bits>(const sru_amd_shape &, const BwdParams &, hipStream_t);
 }  // namespace sru_amd

@@ -1,0 +1,6 @@
+// Backward scan kernels and their launcher for half_bits streams.
+#include "sru_dispatch.h"
+
+namespace sru_amd {
+template void launch_backward<half_bits>(const sru_amd_shape &, const BwdParams &, hipStream_t);
+}  // namespace sru_amd

@@ -1,7 +1,6 @@
-// Scan kernels and their launchers for float streams.
+// Forward scan kernels and their launcher for float streams.
 #include "sru_dispatch.h"
 
 namespace sru_amd {
 template void launch_forward<float>(const sru_amd_shape &, const FwdParams &, hipStream_t);
-template void launch_backward<float>(const sru_amd_shape &, const BwdParams &, hipStream_t);
 }  // namespace sru_amd

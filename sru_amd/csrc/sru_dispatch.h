@@ -1,4 +1,4 @@
-// Kernel selection for one stream element type T. Included by scan_<type>.hip only.
+// Kernel selection for one stream element type T. Included by scan_<type>_fwd.hip and scan_<type>_bwd.hip only.
 //
 // Fast kernels exist for the two layouts the SRU layer produces with a skip term and no
 // per-step weight_c: (k=3, skip from x) and (k=4, skip from U[..., 3]); whether a padding

@@ -1,5 +1,5 @@
 // Host-side launchers of the scan kernels, one explicit instantiation per stream element
-// type (scan_f32.hip, scan_f16.hip, scan_bf16.hip) so the three compile in parallel.
+// type and pass (scan_f32_fwd.hip, scan_f32_bwd.hip, ... scan_bf16_bwd.hip) so the six compile in parallel.
 #pragma once
 
 #include <hip/hip_runtime.h>
