@@ -217,8 +217,8 @@ def main():
                          "reference does, instead of float checkpoints every 8 steps (the path "
                          "the autograd Function of this package takes)")
     ap.add_argument("--no-skip", action="store_true",
-                    help="side measurement of the general kernels: no skip term (has_skip_term=False; "
-                         "the state after every step is kept, as those kernels need)")
+                    help="side measurement: no skip term (has_skip_term=False); with a k=4 workload this "
+                         "runs the general kernels, which keep the state after every step")
     ap.add_argument("--tanh", action="store_true",
                     help="side measurement: activation_type = tanh (the reference's deprecated use_tanh)")
     ap.add_argument("--graph", action="store_true",
@@ -251,7 +251,7 @@ def main():
     tdt = TORCH_DT[args.dtype]
     es = DT_BYTES[args.dtype]
     lib = _lib.load()
-    ckpt = not args.full_state and not fwd_only and not args.no_skip
+    ckpt = not args.full_state and not fwd_only and not (args.no_skip and k == 4)
     use_x = k == 3 and not args.no_skip      # the skip term is read from x
     if args.tanh:
         name += " tanh"

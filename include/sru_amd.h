@@ -82,8 +82,8 @@ typedef struct sru_amd_shape {
                               * SRU_AMD_STATE_INTERVAL: float checkpoints only, one row per
                               *   SRU_AMD_STATE_INTERVAL steps of each column's walk,
                               *   (max(1, L / SRU_AMD_STATE_INTERVAL), B, D') float; the backward
-                              *   call rebuilds the states in between. Needs is_custom 0 and a
-                              *   skip term. No counterpart in the reference. */
+                              *   call rebuilds the states in between. Needs is_custom 0 and,
+                              *   with k = 4, a skip term. No counterpart in the reference. */
 } sru_amd_shape;
 
 #define SRU_AMD_STATE_INTERVAL 8

@@ -35,7 +35,8 @@ int check_shape(const sru_amd_shape *s) {
     if (s->state_interval != 0 && s->state_interval != 1 && s->state_interval != SRU_AMD_STATE_INTERVAL)
         return SRU_AMD_ERR_BAD_FLAGS;
     // checkpointed state exists only for the fast kernels
-    if (s->state_interval == SRU_AMD_STATE_INTERVAL && (s->is_custom != 0 || s->skip_type == 0))
+    if (s->state_interval == SRU_AMD_STATE_INTERVAL &&
+        (s->is_custom != 0 || (s->skip_type == 0 && s->k == 4)))
         return SRU_AMD_ERR_BAD_FLAGS;
     // D' must fit an int, the grid must fit 2^31-1 workgroups and the largest stream
     // (L*B*D'*k elements) must stay far inside the 64-bit byte offsets the kernels use.

@@ -1,9 +1,10 @@
 // Kernel selection for one stream element type T. Included by scan_<type>_fwd.hip and scan_<type>_bwd.hip only.
 //
-// Fast kernels exist for the two layouts the SRU layer produces with a skip term and no
-// per-step weight_c: (k=3, skip from x) and (k=4, skip from U[..., 3]); whether a padding
-// mask is given, whether and how c is stored and the activation are compiled in. Everything
-// else (per-step weight_c, no skip term) runs the general kernels, one column per lane.
+// Fast kernels exist for the three layouts the SRU layer produces without a per-step
+// weight_c: (k=3, skip from x), (k=3, no skip term) and (k=4, skip from U[..., 3]); whether a
+// padding mask is given, whether and how c is stored and the activation are compiled in.
+// Everything else (per-step weight_c; k=4 without a skip term, which the layer never
+// produces) runs the general kernels, one column per lane.
 #pragma once
 
 #include "sru_launch.h"
@@ -184,12 +185,13 @@ void pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
 // (k, skip_type) pairs that pass the shape check: (3,0) (3,1) (4,0) (4,2).
 template <typename T>
 void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
-    const bool general = s.is_custom != 0 || s.skip_type == 0;
+    const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
     const dim3 grid = grid_for(p.ncols, 1), block(kBlock);
     constexpr int P = kGeneralDepth;
     if (!general) {
-        if (s.k == 3) pick_forward<T, 3, 1>(s, p, st);
-        else pick_forward<T, 4, 2>(s, p, st);
+        if (s.k == 4) pick_forward<T, 4, 2>(s, p, st);
+        else if (s.skip_type == 1) pick_forward<T, 3, 1>(s, p, st);
+        else pick_forward<T, 3, 0>(s, p, st);
     } else if (s.k == 3 && s.skip_type == 1) {
         hipLaunchKernelGGL((forward_scan<T, 3, 1, kGeneral | kFwdNt, 1, P>), grid, block, 0, st, p);
     } else if (s.k == 3) {
@@ -203,12 +205,13 @@ void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) 
 
 template <typename T>
 void launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
-    const bool general = s.is_custom != 0 || s.skip_type == 0;
+    const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
     const dim3 grid = grid_for(p.ncols, 1), block(kBlock);
     constexpr int P = kGeneralDepth;
     if (!general) {
-        if (s.k == 3) pick_backward<T, 3, 1>(s, p, st);
-        else pick_backward<T, 4, 2>(s, p, st);
+        if (s.k == 4) pick_backward<T, 4, 2>(s, p, st);
+        else if (s.skip_type == 1) pick_backward<T, 3, 1>(s, p, st);
+        else pick_backward<T, 3, 0>(s, p, st);
     } else if (s.k == 3 && s.skip_type == 1) {
         hipLaunchKernelGGL((backward_scan<T, 3, 1, kGeneral | kBwdNt, 1, P>), grid, block, 0, st, p);
     } else if (s.k == 3) {

@@ -572,9 +572,14 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
                     const float g1 = sigmoid(uu[c * K + 1] + wc1[c] * cur[c] + b1[c]);
                     const float g2 = sigmoid(uu[c * K + 2] + wc2[c] * cur[c] + b2[c]);
                     const float cn = (cur[c] - u0) * g1 + u0;
-                    const float xv = (SKIP == 1) ? xx[c] * sx : uu[c * K + K - 1];
                     const float val = TANH ? tanh_fast(cn) : cn;
-                    const float out = (val - xv) * m[c] * g2 + xv;
+                    float out;
+                    if constexpr (SKIP != 0) {
+                        const float xv = (SKIP == 1) ? xx[c] * sx : uu[c * K + K - 1];
+                        out = (val - xv) * m[c] * g2 + xv;
+                    } else {
+                        out = val * m[c] * g2;
+                    }
                     cur[c] = padded ? cur[c] : cn;
                     hv[c] = padded ? 0.0f : out;
                     cv[c] = cur[c];
@@ -928,7 +933,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                     const float dact = TANH ? (1.0f - val * val) : 1.0f;
                     const float u0 = u0s[i][c];
                     const float G1 = g1[i][c], G2 = g2[i][c];
-                    const float xv = (SKIP == 1) ? xx[c] * sx : xs[i][c];
+                    const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? xx[c] * sx : xs[i][c];
                     const float gh = ghs[c];
 
                     const float gg2 = gh * (val - xv) * m[c] * (G2 * (1.0f - G2));

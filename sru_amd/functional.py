@@ -76,9 +76,10 @@ class _Problem:
         self.dtype = u.dtype
         self.squeeze = x.dim() == 2
         # Between forward and backward keep float checkpoints of the state instead of the
-        # state after every step wherever the kernels support it (no per-step weight_c, a
-        # skip term): the backward kernel rebuilds what lies in between.
-        self.checkpointed = bool(checkpoint_state and not self.is_custom and self.skip_type != 0)
+        # state after every step wherever the kernels support it (no per-step weight_c; with
+        # four streams, a skip term): the backward kernel rebuilds what lies in between.
+        self.checkpointed = bool(checkpoint_state and not self.is_custom
+                                 and not (self.skip_type == 0 and self.k == 4))
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
                                 activation_type, self.skip_type, self.is_custom,
                                 _DTYPES[u.dtype],
