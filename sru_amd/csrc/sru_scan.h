@@ -335,6 +335,21 @@ constexpr int kUniform = 128;// MODE bit (chunked fast kernels): a wavefront lie
 // from its checkpoint while it holds the chunk's U in registers anyway.
 constexpr int kCkptInterval = 8;
 
+// Workgroup index used for the column mapping. Workgroups are dealt to the 8 XCDs round-robin
+// (workgroup i runs on XCD i % 8); SRU_AMD_XCD_REMAP = 1 renumbers them so that every XCD owns
+// one contiguous eighth of the columns (tuning builds; 0 = identity).
+#ifndef SRU_AMD_XCD_REMAP
+#define SRU_AMD_XCD_REMAP 0
+#endif
+__device__ __forceinline__ uint32_t workgroup_index() {
+#if SRU_AMD_XCD_REMAP
+    const uint32_t n = gridDim.x, b = blockIdx.x;
+    return (n % 8 == 0) ? (b % 8) * (n / 8) + b / 8 : b;
+#else
+    return blockIdx.x;
+#endif
+}
+
 // ================================================================= forward scan
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
 // U[..., 3]. COLS: columns per lane (2 needs an even d). P: ring depth.
@@ -498,13 +513,14 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
-    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
+    const uint32_t wg = workgroup_index();
+    const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;  // columns of a pair are col - q, col - q + 1
 
     // colu decides direction and batch row: the wavefront's first column when that is the same
     // for all its lanes (scalar), else the lane's own column
-    const int64_t colu = UNI ? (int64_t)blockIdx.x * (kBlock * COLS) : col;
+    const int64_t colu = UNI ? (int64_t)wg * (kBlock * COLS) : col;
     const uint32_t lane = (uint32_t)(col - colu);
     const int Dp = p.Dp;
     const int ju = (int)(colu % Dp);
@@ -826,11 +842,12 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
-    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
+    const uint32_t wg = workgroup_index();
+    const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;
 
-    const int64_t colu = UNI ? (int64_t)blockIdx.x * (kBlock * COLS) : col;  // see forward_scan_chunked
+    const int64_t colu = UNI ? (int64_t)wg * (kBlock * COLS) : col;  // see forward_scan_chunked
     const uint32_t lane = (uint32_t)(col - colu);
     const int Dp = p.Dp;
     const int ju = (int)(colu % Dp);
