@@ -336,15 +336,21 @@ constexpr int kUniform = 128;// MODE bit (chunked fast kernels): a wavefront lie
 constexpr int kCkptInterval = 8;
 
 // Workgroup index used for the column mapping. Workgroups are dealt to the 8 XCDs round-robin
-// (workgroup i runs on XCD i % 8); SRU_AMD_XCD_REMAP = 1 renumbers them so that every XCD owns
-// one contiguous eighth of the columns (tuning builds; 0 = identity).
+// (workgroup i runs on XCD i % 8); SRU_AMD_XCD_REMAP renumbers them so that every XCD owns one
+// contiguous eighth of the columns (1) or of the hidden indices of every batch row (2). Both
+// measured no better than the identity (0), which is the default; the others serve tuning builds.
 #ifndef SRU_AMD_XCD_REMAP
 #define SRU_AMD_XCD_REMAP 0
 #endif
-__device__ __forceinline__ uint32_t workgroup_index() {
-#if SRU_AMD_XCD_REMAP
+__device__ __forceinline__ uint32_t workgroup_index(uint32_t groups_per_row = 0) {
+#if SRU_AMD_XCD_REMAP == 1
     const uint32_t n = gridDim.x, b = blockIdx.x;
     return (n % 8 == 0) ? (b % 8) * (n / 8) + b / 8 : b;
+#elif SRU_AMD_XCD_REMAP == 2   // every XCD owns one contiguous eighth of the hidden indices of every batch row
+    const uint32_t G = groups_per_row, b = blockIdx.x;
+    if (G == 0 || G % 8 != 0) return b;
+    const uint32_t x = b % 8, i = b / 8, per = G / 8;
+    return (i / per) * G + x * per + i % per;
 #else
     return blockIdx.x;
 #endif
@@ -513,7 +519,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
-    const uint32_t wg = workgroup_index();
+    const uint32_t wg = workgroup_index(UNI ? (uint32_t)(p.Dp / (kBlock * COLS)) : 0u);
     const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;  // columns of a pair are col - q, col - q + 1
@@ -842,7 +848,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
-    const uint32_t wg = workgroup_index();
+    const uint32_t wg = workgroup_index(UNI ? (uint32_t)(p.Dp / (kBlock * COLS)) : 0u);
     const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;
