@@ -18,7 +18,7 @@ import torch.nn as nn
 from torch import Tensor
 from torch.nn.utils.rnn import PackedSequence, pad_packed_sequence, pack_padded_sequence
 
-from .ops import elementwise_recurrence_gpu, elementwise_recurrence_inference
+from .ops import elementwise_recurrence_gpu
 
 
 class SRUCell(nn.Module):
@@ -29,8 +29,15 @@ class SRUCell(nn.Module):
                  use_tanh: bool = False, highway_bias: float = 0.0, has_skip_term: bool = True,
                  layer_norm: bool = False, rescale: bool = True, v1: bool = False,
                  custom_m: Optional[nn.Module] = None, amp_recurrence_fp16: bool = False,
-                 normalize_after: bool = False, weight_c_init: Optional[float] = None):
+                 normalize_after: bool = False, weight_c_init: Optional[float] = None,
+                 native_16bit: bool = True):
+        """Arguments as sru/modules.py:32-50. `native_16bit` (no counterpart there): under
+        autocast, or with 16-bit inputs, the kernels read a float16 / bfloat16 U as it is and
+        return h in that dtype (state and arithmetic stay float32); False restores the
+        reference's policy of casting U and x to float32 first and returning a float32 h
+        (sru/ops.py:116-127)."""
         super().__init__()
+        self.native_16bit = native_16bit
         self.input_size = input_size
         self.hidden_size = hidden_size                       # per direction
         self.bidirectional = bidirectional
@@ -141,12 +148,12 @@ class SRUCell(nn.Module):
     def apply_recurrence(self, U: Tensor, V: Tensor, residual: Tensor, c0: Tensor,
                          scale_val: Optional[Tensor], mask_c: Optional[Tensor],
                          mask_pad: Optional[Tensor]) -> List[Tensor]:
-        """Same call as sru/modules.py:296-318, minus the CPU branches."""
-        args = (U, residual, V, self.bias, c0, self.activation_type, self.hidden_size,
-                self.bidirectional, self.has_skip_term, scale_val, mask_c, mask_pad)
-        if torch.is_grad_enabled():
-            return elementwise_recurrence_gpu(*args, self.amp_recurrence_fp16)
-        return elementwise_recurrence_inference(*args)
+        """The call of sru/modules.py:296-304: always the training entry, which itself skips the
+        state store when nothing can be differentiated. There are no CPU branches."""
+        return elementwise_recurrence_gpu(
+            U, residual, V, self.bias, c0, self.activation_type, self.hidden_size,
+            self.bidirectional, self.has_skip_term, scale_val, mask_c, mask_pad,
+            self.amp_recurrence_fp16, getattr(self, "native_16bit", True))
 
     def compute_UV(self, input: Tensor, c0: Optional[Tensor],
                    mask_pad: Optional[Tensor]) -> Tuple[Tensor, Tensor]:
@@ -178,23 +185,37 @@ class SRUCell(nn.Module):
         return self.bias.new_empty(size).bernoulli_(1 - p).div_(1 - p)
 
     def extra_repr(self):
+        # the fields and order of sru/modules.py:388-413
         parts = [f"{self.input_size}, {self.hidden_size}"]
-        if self.projection_size:
+        if self.projection_size > 0:
             parts.append(f"projection_size={self.projection_size}")
         if self.dropout > 0:
             parts.append(f"dropout={self.dropout}")
+        if self.rnn_dropout > 0:
+            parts.append(f"rnn_dropout={self.rnn_dropout}")
         if self.bidirectional:
-            parts.append("bidirectional=True")
+            parts.append(f"bidirectional={self.bidirectional}")
         if self.highway_bias != 0:
             parts.append(f"highway_bias={self.highway_bias}")
-        if self.activation_type:
+        if self.activation_type != 0:
             parts.append(f"activation={self.activation}")
+        if self.v1:
+            parts.append(f"v1={self.v1}")
         parts.append(f"rescale={self.rescale}")
         if not self.has_skip_term:
-            parts.append("has_skip_term=False")
+            parts.append(f"has_skip_term={self.has_skip_term}")
         if self.layer_norm is not None:
             parts.append("layer_norm=True")
-        return ", ".join(parts)
+        s = ", ".join(parts)
+        if self.custom_m is not None:
+            s += ",\n  custom_m=" + str(self.custom_m)
+        return s
+
+    def __repr__(self):
+        s = self.extra_repr()
+        if len(s.split("\n")) == 1:
+            return "{}({})".format(self.__class__.__name__, s)
+        return "{}({}\n)".format(self.__class__.__name__, s)
 
 
 class SRU(nn.Module):
@@ -207,7 +228,9 @@ class SRU(nn.Module):
                  nn_rnn_compatible_return: bool = False,
                  custom_m: Optional[Union[nn.Module, List[nn.Module]]] = None,
                  proj_input_to_hidden_first: bool = False, amp_recurrence_fp16: bool = False,
-                 normalize_after: bool = False, weight_c_init: Optional[float] = None):
+                 normalize_after: bool = False, weight_c_init: Optional[float] = None,
+                 native_16bit: bool = True):
+        """Arguments as sru/modules.py:437-457; `native_16bit` as in SRUCell."""
         super().__init__()
         self.input_size = input_size
         self.hidden_size = hidden_size
@@ -247,7 +270,7 @@ class SRU(nn.Module):
                 use_tanh=use_tanh, layer_norm=layer_norm, highway_bias=highway_bias,
                 has_skip_term=has_skip_term, rescale=rescale, v1=v1, custom_m=m_i,
                 amp_recurrence_fp16=amp_recurrence_fp16, normalize_after=normalize_after,
-                weight_c_init=weight_c_init))
+                weight_c_init=weight_c_init, native_16bit=native_16bit))
 
     def forward(self, input: Union[Tensor, PackedSequence], c0: Optional[Tensor] = None,
                 mask_pad: Optional[Tensor] = None) -> Tuple[Union[Tensor, PackedSequence], Tensor]:
@@ -288,3 +311,32 @@ class SRU(nn.Module):
             layer.reset_parameters()
         if self.input_to_hidden is not None:
             self.input_to_hidden.reset_parameters()
+
+    def make_backward_compatible(self):
+        """Brings a module object unpickled from an older release up to the current attribute
+        names (sru/modules.py:660-689): releases up to 2.1.7 called the sizes n_in / n_out /
+        out_size / depth / n_proj and the stream count k, had no layer norm that can be carried
+        over, and knew weight norm and relu / selu, which no longer exist; releases up to 2.1.9
+        had neither `input_to_hidden` nor `custom_m`."""
+        self.nn_rnn_compatible_return = getattr(self, "nn_rnn_compatible_return", False)
+        if hasattr(self, "n_in"):
+            if len(self.ln_lst):
+                raise Exception("Layer norm is not backward compatible for sru<=2.1.7")
+            if self.use_weight_norm:
+                raise Exception("Weight norm removed in sru>=2.1.9")
+            self.input_size, self.hidden_size = self.n_in, self.n_out
+            self.output_size, self.num_layers = self.out_size, self.depth
+            self.projection_size = self.n_proj
+            self.use_layer_norm = False
+            for cell in self.rnn_lst:
+                cell.input_size, cell.hidden_size = cell.n_in, cell.n_out
+                cell.output_size = cell.n_out * (2 if cell.bidirectional else 1)
+                cell.num_matrices = cell.k
+                cell.projection_size = cell.n_proj
+                cell.layer_norm = None
+                if cell.activation_type > 1:
+                    raise Exception("ReLU or SeLU activation removed in sru>=2.1.9")
+        if not hasattr(self, "input_to_hidden"):
+            self.input_to_hidden = None
+            for cell in self.rnn_lst:
+                cell.custom_m = None

@@ -32,6 +32,17 @@ def elementwise_recurrence_gpu(U: Tensor, x: Tensor, weight_c: Tensor, bias: Ten
         U, x = U.float(), x.float()
         if weight_c.dim() > 1:
             weight_c = weight_c.float()
+    wants_grad = torch.is_grad_enabled() and any(
+        t.requires_grad for t in (U, x, weight_c, bias, c_init))
+    if not wants_grad:
+        # Nothing will be differentiated (torch.no_grad(), or no input requires grad): same
+        # results as the autograd Function, dropout mask included (the reference takes this
+        # branch of sru/modules.py:296-304 for training-mode modules under no_grad as well),
+        # without storing the state for a backward pass that cannot come.
+        h, last_hidden, _ = elementwise_recurrence_forward(
+            U, x, weight_c, bias, c_init, activation_type, hidden_size, bidirectional,
+            has_skip_term, scale_x, dropout_mask_c, mask_pad, keep_c=False)
+        return h, last_hidden
     return ElementwiseRecurrence.apply(U, x, weight_c, bias, c_init, activation_type,
                                        hidden_size, bidirectional, has_skip_term, scale_x,
                                        dropout_mask_c, mask_pad)

@@ -201,3 +201,34 @@ def test_training_steps_with_and_without_autocast(amp_dtype):
         opt.step()
         losses.append(float(loss.detach()))
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
+
+
+@pytest.mark.parametrize("amp", [None, torch.bfloat16], ids=["fp32", "bf16_autocast"])
+def test_training_mode_under_no_grad_uses_the_dropout_mask(amp):
+    # sru/modules.py:296-304 takes the training entry whenever the module is not scripted, so a
+    # module in train() mode under torch.no_grad() draws and applies its dropout mask; the output
+    # must equal the grad-enabled run with the same seed
+    torch.manual_seed(11)
+    model = SRU(64, 64, num_layers=3, dropout=0.3, bidirectional=True, rescale=True).to(DEV).train()
+    x = torch.randn(20, 5, 64, device=DEV)
+
+    def run():
+        torch.manual_seed(99)
+        with torch.autocast("cuda", dtype=amp, enabled=amp is not None):
+            return model(x)
+
+    h_grad, c_grad = run()
+    with torch.no_grad():
+        h_ng, c_ng = run()
+    assert h_grad.requires_grad and not h_ng.requires_grad
+    assert torch.equal(h_grad.detach(), h_ng) and torch.equal(c_grad.detach(), c_ng)
+    model.eval()
+    with torch.no_grad():
+        h_eval, _ = run()
+    assert not torch.equal(h_eval, h_ng)          # the mask was really applied
+    # inputs that need no gradient at all (frozen parameters) take the same path with grad enabled
+    model.train()
+    for p in model.parameters():
+        p.requires_grad_(False)
+    h_frozen, _ = run()
+    assert torch.equal(h_frozen, h_ng)

@@ -95,3 +95,87 @@ def test_error_behaviour():
             return x
     with pytest.raises(ValueError):
         SRUCell(4, 4, custom_m=Bad()).compute_UV(torch.zeros(3, 2, 4), None, None)
+
+
+def test_repr_follows_the_reference_format():
+    # sru/modules.py:384-419
+    assert repr(SRUCell(8, 8)) == "SRUCell(8, 8, rescale=True)"
+    cell = SRUCell(16, 8, dropout=0.1, rnn_dropout=0.2, bidirectional=True, n_proj=4, use_tanh=True,
+                   highway_bias=-1.0, has_skip_term=False, layer_norm=True, rescale=False, v1=True)
+    assert repr(cell) == ("SRUCell(16, 8, projection_size=4, dropout=0.1, rnn_dropout=0.2, bidirectional=True, "
+                          "highway_bias=-1.0, activation=tanh, v1=True, rescale=False, has_skip_term=False, "
+                          "layer_norm=True)")
+    with_m = SRUCell(4, 4, custom_m=torch.nn.Linear(4, 12, bias=False))
+    assert repr(with_m) == ("SRUCell(4, 4, rescale=True,\n  custom_m=Linear(in_features=4, out_features=12, "
+                            "bias=False)\n)")
+    assert "SRUCell(4, 4, rescale=False)" in repr(SRU(4, 4))
+
+
+def _drop(module, name):
+    """Removes an attribute wherever nn.Module keeps it (plain attribute or sub-module slot)."""
+    if name in module._modules:
+        del module._modules[name]
+    else:
+        module.__dict__.pop(name, None)
+
+
+def test_make_backward_compatible():
+    # sru/modules.py:660-689: attribute names of releases <= 2.1.7 and <= 2.1.9
+    model = SRU(6, 5, num_layers=2, bidirectional=True, projection_size=2)
+    # an object as release 2.1.7 pickled it: old names only
+    old = SRU(6, 5, num_layers=2, bidirectional=True, projection_size=2)
+    old.n_in, old.n_out, old.out_size, old.depth, old.n_proj = 6, 5, 10, 2, 2
+    old.ln_lst, old.use_weight_norm = [], False
+    for name in ("input_size", "hidden_size", "output_size", "num_layers", "projection_size", "use_layer_norm",
+                 "nn_rnn_compatible_return"):
+        delattr(old, name)
+    _drop(old, "input_to_hidden")
+    for cell in old.rnn_lst:
+        cell.n_in, cell.n_out, cell.k, cell.n_proj = cell.input_size, cell.hidden_size, cell.num_matrices, 2
+        for name in ("input_size", "hidden_size", "output_size", "num_matrices", "projection_size", "custom_m",
+                     "layer_norm"):
+            _drop(cell, name)
+    old.make_backward_compatible()
+    for name in ("input_size", "hidden_size", "output_size", "num_layers", "projection_size"):
+        assert getattr(old, name) == getattr(model, name), name
+    assert old.use_layer_norm is False and old.nn_rnn_compatible_return is False
+    assert old.input_to_hidden is None
+    for cell, new in zip(old.rnn_lst, model.rnn_lst):
+        for name in ("input_size", "hidden_size", "output_size", "num_matrices", "projection_size"):
+            assert getattr(cell, name) == getattr(new, name), name
+        assert cell.layer_norm is None and cell.custom_m is None
+    # what cannot be carried over is refused
+    old.use_weight_norm = True
+    with pytest.raises(Exception, match="Weight norm"):
+        old.make_backward_compatible()
+    old.use_weight_norm, old.ln_lst = False, [1]
+    with pytest.raises(Exception, match="Layer norm"):
+        old.make_backward_compatible()
+    old.ln_lst = []
+    old.rnn_lst[0].activation_type = 2
+    with pytest.raises(Exception, match="ReLU or SeLU"):
+        old.make_backward_compatible()
+    # a current object passes through unchanged
+    before = dict(model.__dict__)
+    model.make_backward_compatible()
+    assert {k: v for k, v in model.__dict__.items() if k != "_modules"} == \
+        {k: v for k, v in before.items() if k != "_modules"}
+
+
+def test_large_stack_restatement_equals_the_python_loop_restatement():
+    # tests/stack_ref.py: the float64 stack built on the C oracle (used at sizes where the Python
+    # loop is too slow) must agree with the one built on the differentiable torch loop
+    from tests.stack_ref import stack_forward, stack_forward_large
+    torch.manual_seed(4)
+    model = SRU(6, 8, num_layers=3, bidirectional=True, layer_norm=True, rescale=True, projection_size=3,
+                dropout=0.2)
+    x = torch.randn(9, 4, 6)
+    pad = torch.arange(9)[:, None] >= torch.tensor([9, 4, 7, 1])[None, :]
+    h1, c1, p1 = stack_forward(model, x, mask_pad=pad)
+    h2, c2, p2 = stack_forward_large(model, x, mask_pad=pad, device="cpu")
+    probe = torch.randn(h1.shape, dtype=torch.float64)
+    (h1 * probe).sum().backward()
+    (h2 * probe).sum().backward()
+    assert float((h1 - h2).abs().max()) <= 1e-12 and float((c1 - c2).abs().max()) <= 1e-12
+    for n in p1:
+        assert float((p1[n].grad - p2[n].grad).abs().max()) <= 1e-10 * max(1.0, float(p1[n].grad.abs().max())), n
