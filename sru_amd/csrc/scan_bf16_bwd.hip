@@ -2,5 +2,5 @@
 #include "sru_dispatch.h"
 
 namespace sru_amd {
-template void launch_backward<bf16_bits>(const sru_amd_shape &, const BwdParams &, hipStream_t);
+template hipError_t launch_backward<bf16_bits>(const sru_amd_shape &, const BwdParams &, hipStream_t);
 }  // namespace sru_amd

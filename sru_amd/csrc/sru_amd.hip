@@ -49,6 +49,48 @@ int check_shape(const sru_amd_shape *s) {
     return SRU_AMD_OK;
 }
 
+// The backward call after the shape and workspace checks: pointer checks, then the
+// scan and the batch reduction enqueued on `stream`, with the per-column partial sums in
+// `partial` (4 * B * D' floats of device memory).
+int backward_core(const sru_amd_shape *shape, const void *u, const void *x, const void *weight_c,
+                  const float *bias, const float *c_init, const float *mask_c, const uint8_t *mask_pad,
+                  const float *scale_x, const void *c, const void *grad_h, const float *grad_last,
+                  void *grad_u, void *grad_x, void *grad_wc, float *grad_bias, float *grad_init,
+                  float *partial, void *stream) {
+    const sru_amd_shape &s = *shape;
+    if (!u || !weight_c || !bias || !c_init || !c || !grad_h || !grad_last || !grad_u || !grad_wc ||
+        !grad_bias || !grad_init)
+        return SRU_AMD_ERR_NULL_POINTER;
+    if (s.skip_type == 1 && (!x || !grad_x)) return SRU_AMD_ERR_NULL_POINTER;
+    const size_t es = elem_size(s.dtype);
+    const size_t group = (s.k == 4) ? 4 * es : es;
+    const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
+    if (!aligned(u, group) || !aligned(grad_u, group) || !aligned(c, ckpt ? 4 : es) || !aligned(grad_h, es) ||
+        (s.skip_type == 1 && (!aligned(x, es) || !aligned(grad_x, es))) ||
+        !aligned(weight_c, s.is_custom ? 2 * es : 4) || !aligned(grad_wc, s.is_custom ? 2 * es : 4) ||
+        !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(grad_last, 4) || !aligned(grad_bias, 4) ||
+        !aligned(grad_init, 4) || (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
+        return SRU_AMD_ERR_MISALIGNED;
+
+    BwdParams p{};
+    p.u = u; p.x = x; p.wc = weight_c; p.bias = bias; p.c0 = c_init; p.mask_c = mask_c;
+    p.pad = mask_pad; p.scale_x = scale_x; p.gh = grad_h; p.glast = grad_last;
+    p.c = ckpt ? nullptr : c;
+    p.ckpt = ckpt ? static_cast<const float *>(c) : nullptr;
+    p.gu = grad_u; p.gx = grad_x; p.gwc_steps = s.is_custom ? grad_wc : nullptr;
+    p.ginit = grad_init; p.partial = partial;
+    p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
+    p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const hipError_t err = s.dtype == SRU_AMD_F32   ? launch_backward<float>(s, p, st)
+                           : s.dtype == SRU_AMD_F16 ? launch_backward<half_bits>(s, p, st)
+                                                    : launch_backward<bf16_bits>(s, p, st);
+    if (err != hipSuccess) return SRU_AMD_ERR_LAUNCH;
+    return launch_reduce(p.partial, s.is_custom ? nullptr : static_cast<float *>(grad_wc), grad_bias, p.B,
+                         p.Dp, st) == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" {
@@ -95,11 +137,10 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
     p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
-    (void)hipGetLastError();
-    if (s.dtype == SRU_AMD_F32) launch_forward<float>(s, p, st);
-    else if (s.dtype == SRU_AMD_F16) launch_forward<half_bits>(s, p, st);
-    else launch_forward<bf16_bits>(s, p, st);
-    return hipGetLastError() == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+    const hipError_t err = s.dtype == SRU_AMD_F32   ? launch_forward<float>(s, p, st)
+                           : s.dtype == SRU_AMD_F16 ? launch_forward<half_bits>(s, p, st)
+                                                    : launch_forward<bf16_bits>(s, p, st);
+    return err == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
 }
 
 size_t sru_amd_state_bytes(const sru_amd_shape *shape) {
@@ -124,45 +165,11 @@ int sru_amd_backward(const sru_amd_shape *shape, const void *u, const void *x, c
                      void *grad_wc, float *grad_bias, float *grad_init, void *workspace,
                      size_t workspace_bytes, void *stream) {
     if (const int rc = check_shape(shape)) return rc;
-    const sru_amd_shape &s = *shape;
-    if (!u || !weight_c || !bias || !c_init || !c || !grad_h || !grad_last || !grad_u || !grad_wc ||
-        !grad_bias || !grad_init)
-        return SRU_AMD_ERR_NULL_POINTER;
-    if (s.skip_type == 1 && (!x || !grad_x)) return SRU_AMD_ERR_NULL_POINTER;
-    const size_t es = elem_size(s.dtype);
-    const size_t group = (s.k == 4) ? 4 * es : es;
-    const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
-    if (!aligned(u, group) || !aligned(grad_u, group) || !aligned(c, ckpt ? 4 : es) || !aligned(grad_h, es) ||
-        (s.skip_type == 1 && (!aligned(x, es) || !aligned(grad_x, es))) ||
-        !aligned(weight_c, s.is_custom ? 2 * es : 4) || !aligned(grad_wc, s.is_custom ? 2 * es : 4) ||
-        !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(grad_last, 4) || !aligned(grad_bias, 4) ||
-        !aligned(grad_init, 4) || (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
-        return SRU_AMD_ERR_MISALIGNED;
     if (!workspace || !aligned(workspace, 16) ||
         workspace_bytes < sru_amd_backward_workspace_bytes(shape))
         return SRU_AMD_ERR_WORKSPACE;
-
-    BwdParams p{};
-    p.u = u; p.x = x; p.wc = weight_c; p.bias = bias; p.c0 = c_init; p.mask_c = mask_c;
-    p.pad = mask_pad; p.scale_x = scale_x; p.gh = grad_h; p.glast = grad_last;
-    p.c = ckpt ? nullptr : c;
-    p.ckpt = ckpt ? static_cast<const float *>(c) : nullptr;
-    p.gu = grad_u; p.gx = grad_x; p.gwc_steps = s.is_custom ? grad_wc : nullptr;
-    p.ginit = grad_init; p.partial = static_cast<float *>(workspace);
-    p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
-    p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
-
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    (void)hipGetLastError();
-    if (s.dtype == SRU_AMD_F32) launch_backward<float>(s, p, st);
-    else if (s.dtype == SRU_AMD_F16) launch_backward<half_bits>(s, p, st);
-    else launch_backward<bf16_bits>(s, p, st);
-    if (hipGetLastError() != hipSuccess) return SRU_AMD_ERR_LAUNCH;
-
-    const dim3 rgrid((unsigned)((p.Dp + 63) / 64), 4);
-    hipLaunchKernelGGL(reduce_partials, rgrid, dim3(64 * kReduceSlices), 0, st, p.partial,
-                       s.is_custom ? nullptr : static_cast<float *>(grad_wc), grad_bias, p.B, p.Dp);
-    return hipGetLastError() == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+    return backward_core(shape, u, x, weight_c, bias, c_init, mask_c, mask_pad, scale_x, c, grad_h, grad_last,
+                         grad_u, grad_x, grad_wc, grad_bias, grad_init, static_cast<float *>(workspace), stream);
 }
 
 }  // extern "C"

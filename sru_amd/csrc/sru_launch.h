@@ -9,10 +9,11 @@
 
 namespace sru_amd {
 
+// Both return the status of the launch itself (hipSuccess = enqueued).
 template <typename T>
-void launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t stream);
+hipError_t launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t stream);
 
 template <typename T>
-void launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t stream);
+hipError_t launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t stream);
 
 }  // namespace sru_amd

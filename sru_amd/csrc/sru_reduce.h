@@ -46,4 +46,11 @@ reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t 
     }
 }
 
+inline hipError_t launch_reduce(const float *partial, float *grad_wc, float *grad_bias, int64_t B, int32_t Dp,
+                                hipStream_t st) {
+    void *args[] = {&partial, &grad_wc, &grad_bias, &B, &Dp};
+    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_partials), dim3((unsigned)((Dp + 63) / 64), 4),
+                           dim3(64 * kReduceSlices), args, 0, st);
+}
+
 }  // namespace sru_amd

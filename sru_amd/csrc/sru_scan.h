@@ -266,10 +266,25 @@ struct Stream {
 };
 
 // ---------------------------------------------------------------- gate arithmetic
-// sigmoid through the hardware exp2 and reciprocal (1 ulp each): absolute error of the
-// result stays below 2e-7 over the whole real line; saturates cleanly to 0 and 1.
+// sigmoid through the hardware exp2 and reciprocal (1 ulp each). The reciprocal's ulp is the
+// largest part of the error where the gate is close to 1, and the state carries it along the
+// whole walk, so float streams refine it with one Newton step (two fused multiply-adds): the
+// result is then within 1e-7 of the exact sigmoid over the whole real line. 16-bit streams
+// round their outputs to 2^-9 and skip the step. Saturates cleanly to 0 (2^-126) and 1.
+#ifndef SRU_AMD_REFINE_SIGMOID
+#define SRU_AMD_REFINE_SIGMOID 1
+#endif
+template <typename T>
 __device__ __forceinline__ float sigmoid(float v) {
-    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+    if constexpr (sizeof(T) == 4 && SRU_AMD_REFINE_SIGMOID) {
+        // the exponent is capped so that d stays finite (inf * 0 in the correction would be NaN);
+        // at the cap the result is 2^-126
+        const float d = 1.0f + __builtin_amdgcn_exp2f(fminf(-1.4426950408889634f * v, 126.0f));
+        const float r = __builtin_amdgcn_rcpf(d);
+        return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
+    } else {
+        return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+    }
 }
 
 // tanh through the same two units: 1 - 2 / (1 + e^(2v)). Absolute error below 3e-7 over the
@@ -335,26 +350,20 @@ constexpr int kUniform = 128;// MODE bit (chunked fast kernels): a wavefront lie
 // from its checkpoint while it holds the chunk's U in registers anyway.
 constexpr int kCkptInterval = 8;
 
-// Workgroup index used for the column mapping. Workgroups are dealt to the 8 XCDs round-robin
-// (workgroup i runs on XCD i % 8); SRU_AMD_XCD_REMAP renumbers them so that every XCD owns one
-// contiguous eighth of the columns (1) or of the hidden indices of every batch row (2). Both
-// measured no better than the identity (0), which is the default; the others serve tuning builds.
-#ifndef SRU_AMD_XCD_REMAP
-#define SRU_AMD_XCD_REMAP 0
-#endif
-__device__ __forceinline__ uint32_t workgroup_index(uint32_t groups_per_row = 0) {
-#if SRU_AMD_XCD_REMAP == 1
-    const uint32_t n = gridDim.x, b = blockIdx.x;
-    return (n % 8 == 0) ? (b % 8) * (n / 8) + b / 8 : b;
-#elif SRU_AMD_XCD_REMAP == 2   // every XCD owns one contiguous eighth of the hidden indices of every batch row
-    const uint32_t G = groups_per_row, b = blockIdx.x;
-    if (G == 0 || G % 8 != 0) return b;
-    const uint32_t x = b % 8, i = b / 8, per = G / 8;
-    return (i / per) * G + x * per + i % per;
-#else
-    return blockIdx.x;
-#endif
-}
+// Kahan-compensated accumulation of one chunk's (or ring round's) sum `part` into a running sum
+// that lives over the whole walk: the running sums of the weight_c / bias gradients have
+// L terms per column, and plain float accumulation of that many terms was the largest single
+// contribution to their error. Four instructions per chunk and sum, not per cell.
+struct CompensatedSum {
+    float sum = 0.f, comp = 0.f;
+    __device__ __forceinline__ void add(float part) {
+        const float y = part - comp;
+        const float t = sum + y;
+        comp = (t - sum) - y;
+        sum = t;
+    }
+    __device__ __forceinline__ float value() const { return sum - comp; }
+};
 
 // ================================================================= forward scan
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
@@ -363,8 +372,7 @@ template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
-    constexpr bool CKPT = (MODE & kCkpt) != 0;
-    static_assert(!CKPT || (P == kCkptInterval && !GENERAL), "a ring round is one checkpoint chunk");
+    static_assert((MODE & (kCkpt | kPair | kUniform)) == 0, "those exist in the chunked kernels only");
     const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;  // lane's first column
     if (col >= p.ncols) return;
 
@@ -399,13 +407,6 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     const int64_t ps = flip ? -p.B : p.B;
     T *hp = static_cast<T *>(p.h) + e0;
     T *cp = keep_c ? static_cast<T *>(p.c) + e0 : nullptr;
-    float *kp = CKPT ? p.ckpt + col : nullptr;
-    auto checkpoint = [&]() {  // called after the last step of a chunk
-#pragma unroll
-        for (int c = 0; c < COLS; ++c) kp[c] = cur[c];
-        kp += p.ncols;
-    };
-
     struct Slot {
         Group<T, COLS * K> u;
         Group<T, COLS> x;
@@ -440,8 +441,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             const float u0 = s.u.get(c * K), u1 = s.u.get(c * K + 1), u2 = s.u.get(c * K + 2);
             const float w1 = custom ? s.w.get(2 * c) : wc1[c];
             const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
-            const float g1 = sigmoid(u1 + w1 * cur[c] + b1[c]);
-            const float g2 = sigmoid(u2 + w2 * cur[c] + b2[c]);
+            const float g1 = sigmoid<T>(u1 + w1 * cur[c] + b1[c]);
+            const float g2 = sigmoid<T>(u2 + w2 * cur[c] + b2[c]);
             const float cn = (cur[c] - u0) * g1 + u0;
             const float val = use_tanh ? tanh_fast(cn) : cn;
             float out;
@@ -477,7 +478,6 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             // loads of a round at its end, where none of them has time to land.
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (CKPT) checkpoint();
     }
     for (; s0 < L; s0 += P) {  // last one or two rounds
 #pragma unroll
@@ -488,7 +488,6 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
                 consume(s);
             }
         }
-        if (CKPT && s0 + P <= L) checkpoint();
     }
 #pragma unroll
     for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
@@ -519,7 +518,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
-    const uint32_t wg = workgroup_index(UNI ? (uint32_t)(p.Dp / (kBlock * COLS)) : 0u);
+    const uint32_t wg = blockIdx.x;
     const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;  // columns of a pair are col - q, col - q + 1
@@ -591,8 +590,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float u0 = uu[c * K];
-                    const float g1 = sigmoid(uu[c * K + 1] + wc1[c] * cur[c] + b1[c]);
-                    const float g2 = sigmoid(uu[c * K + 2] + wc2[c] * cur[c] + b2[c]);
+                    const float g1 = sigmoid<T>(uu[c * K + 1] + wc1[c] * cur[c] + b1[c]);
+                    const float g2 = sigmoid<T>(uu[c * K + 2] + wc2[c] * cur[c] + b2[c]);
                     const float cn = (cur[c] - u0) * g1 + u0;
                     const float val = TANH ? tanh_fast(cn) : cn;
                     float out;
@@ -675,7 +674,18 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
 
     float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
     float cur[COLS];  // d loss / d state
-    float gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];
+    float gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];  // sums of the current ring round
+    CompensatedSum sw1[COLS], sw2[COLS], sb1[COLS], sb2[COLS];  // sums over the whole walk
+    auto fold_round = [&]() {
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            sw1[c].add(gw1[c]);
+            sw2[c].add(gw2[c]);
+            sb1[c].add(gb1[c]);
+            sb2[c].add(gb2[c]);
+            gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
+        }
+    };
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         wc1[c] = custom ? 0.f : static_cast<const float *>(p.wc)[j + c];
@@ -755,8 +765,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
             const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
             const float cp = s.first ? c_init[c] : s.cprev.get(c);
             const float u0 = s.u.get(c * K);
-            const float g1 = sigmoid(s.u.get(c * K + 1) + w1 * cp + b1[c]);
-            const float g2 = sigmoid(s.u.get(c * K + 2) + w2 * cp + b2[c]);
+            const float g1 = sigmoid<T>(s.u.get(c * K + 1) + w1 * cp + b1[c]);
+            const float g2 = sigmoid<T>(s.u.get(c * K + 2) + w2 * cp + b2[c]);
             const float val = use_tanh ? tanh_fast(cv[c]) : cv[c];
             const float dact = use_tanh ? (1.0f - val * val) : 1.0f;
             const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
@@ -806,6 +816,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
             fetch(ring[i], s0 + i + P == L - 1);
             __builtin_amdgcn_sched_barrier(0);  // see forward_scan
         }
+        fold_round();
     }
     for (; s0 < L; s0 += P) {
 #pragma unroll
@@ -816,15 +827,16 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
                 consume(s);
             }
         }
+        fold_round();
     }
 
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         p.ginit[col + c] = cur[c];
-        p.partial[col + c] = gw1[c];
-        p.partial[p.ncols + col + c] = gw2[c];
-        p.partial[2 * p.ncols + col + c] = gb1[c];
-        p.partial[3 * p.ncols + col + c] = gb2[c];
+        p.partial[col + c] = sw1[c].value();
+        p.partial[p.ncols + col + c] = sw2[c].value();
+        p.partial[2 * p.ncols + col + c] = sb1[c].value();
+        p.partial[3 * p.ncols + col + c] = sb2[c].value();
     }
 }
 
@@ -843,12 +855,10 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
     // (forward_scan_chunked fetches the flags of a chunk with one load; here, where every flag
     // is needed twice, that measured 0-3 % slower, so the flags stay one load per step)
-    constexpr bool PAD_BY_LANE = false;
     constexpr bool TANH = (MODE & kTanh) != 0;
-    constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
-    const uint32_t wg = workgroup_index(UNI ? (uint32_t)(p.Dp / (kBlock * COLS)) : 0u);
+    const uint32_t wg = blockIdx.x;
     const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
     const int q = PAIR ? (int)(threadIdx.x & 1) : 0;
@@ -862,7 +872,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
 
     float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
     float cur[COLS];  // d loss / d state
-    float gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];
+    CompensatedSum sw1[COLS], sw2[COLS], sb1[COLS], sb2[COLS];  // weight_c / bias gradient sums over the walk
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         wc1[c] = static_cast<const float *>(p.wc)[j + c];
@@ -872,7 +882,6 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
         c_init[c] = p.c0[col + c];
         cur[c] = p.glast[col + c];
-        gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
     }
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
 
@@ -894,7 +903,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         typename SU::G u[TC];
         typename S1::G x[TC];
         typename S1::G gh[TC];
-        uint32_t pad[kPadRegs];  // padding flags of the chunk, see load_chunk
+        uint32_t pad[TC];    // padding flags of the chunk's steps
         float cstart[COLS];  // state before the chunk's first step
     };
 
@@ -908,10 +917,9 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
                 if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
                 k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
-                if (!PAD_BY_LANE) k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
+                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
-        if (PAD_BY_LANE) k.pad[0] = p.pad[pf + (s0 + min((int)(threadIdx.x % TC), n - 1)) * ps];  // see forward_scan_chunked
 #pragma unroll
         for (int c = 0; c < COLS; ++c)
             k.cstart[c] = (ch == 0) ? c_init[c] : p.ckpt[(ch - 1) * p.ncols + col + c];
@@ -924,10 +932,11 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         float u0s[TC][COLS], xs[TC][COLS];  // candidate stream and (k = 4) skip stream, decoded once
 #pragma unroll
         for (int c = 0; c < COLS; ++c) st[0][c] = k.cstart[c];
+        float gw1[COLS] = {}, gw2[COLS] = {}, gb1[COLS] = {}, gb2[COLS] = {};  // this chunk's share of the sums
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
-                const bool padded = (PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i]) != 0;
+                const bool padded = k.pad[i] != 0;
                 float uu[COLS * K];
                 SU::unpack(k.u[i], q, uu);
 #pragma unroll
@@ -935,8 +944,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                     const float cp = st[i][c];
                     u0s[i][c] = uu[c * K];
                     if (SKIP == 2) xs[i][c] = uu[c * K + K - 1];
-                    g1[i][c] = sigmoid(uu[c * K + 1] + wc1[c] * cp + b1[c]);
-                    g2[i][c] = sigmoid(uu[c * K + 2] + wc2[c] * cp + b2[c]);
+                    g1[i][c] = sigmoid<T>(uu[c * K + 1] + wc1[c] * cp + b1[c]);
+                    g2[i][c] = sigmoid<T>(uu[c * K + 2] + wc2[c] * cp + b2[c]);
                     const float cn = (cp - u0s[i][c]) * g1[i][c] + u0s[i][c];
                     st[i + 1][c] = padded ? cp : cn;
                 }
@@ -945,7 +954,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
 #pragma unroll
         for (int i = TC - 1; i >= 0; --i) {
             if (i < n) {
-                const bool padded = (PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i]) != 0;
+                const bool padded = k.pad[i] != 0;
                 float gu[COLS * K], gx[COLS], xx[COLS] = {}, ghs[COLS];
                 if (SKIP == 1) S1::unpack(k.x[i], q, xx);
                 S1::unpack(k.gh[i], q, ghs);
@@ -981,6 +990,13 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 if (SKIP == 1) S1::template store<NTS>(gxbase + e, lane, q, gx);
             }
         }
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) {
+            sw1[c].add(gw1[c]);
+            sw2[c].add(gw2[c]);
+            sb1[c].add(gb1[c]);
+            sb2[c].add(gb2[c]);
+        }
     };
 
     const int64_t nfull = L / TC;
@@ -1014,10 +1030,10 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
         p.ginit[col + c] = cur[c];
-        p.partial[col + c] = gw1[c];
-        p.partial[p.ncols + col + c] = gw2[c];
-        p.partial[2 * p.ncols + col + c] = gb1[c];
-        p.partial[3 * p.ncols + col + c] = gb2[c];
+        p.partial[col + c] = sw1[c].value();
+        p.partial[p.ncols + col + c] = sw2[c].value();
+        p.partial[2 * p.ncols + col + c] = sb1[c].value();
+        p.partial[3 * p.ncols + col + c] = sb2[c].value();
     }
 }
 

@@ -4,7 +4,7 @@ size-independent properties of the domain checked at that size on the GPU alone.
 
 Tolerances: forward outputs 1e-5 absolute; gradient cells 1e-5 * max(1, |reference cell|)
 (absolute 1e-5 for every cell of magnitude up to 1, relative 1e-5 for the few larger ones);
-the sums over L*B = 16384 terms (grad_wc, grad_bias) 1e-5 * max(1, max|reference|). The test
+the sums over L*B = 16384 terms (grad_wc, grad_bias) 1e-6 * max(1, max|reference|). The test
 prints, beside each figure, how far the float32 serial CPU loop itself lands from float64.
 """
 import numpy as np
@@ -62,8 +62,12 @@ def test_headline_shape_against_float64_oracle(checkpointed):
         c_used = to_np(cs)
     gu, gx, gwc, gb, gi = dp.backward()
     g_ref = so.backward(*c.fwd_args(), c_used, c.gh, c.gl, **c.kw())
-    # context: the float32 serial CPU loop (the reference's own arithmetic) against the same float64 result
-    g32 = so.backward(*c.fwd_args(), c_used, c.gh, c.gl, **dict(c.kw(), precision="f32"))
+    # context: the float32 serial CPU loop (the reference's own arithmetic, forward and backward,
+    # working from its own float32 states) against the same float64 result
+    kw32 = dict(c.kw(), precision="f32")
+    h32, c32, _ = so.forward(*c.fwd_args(), **kw32)
+    print(f"float32 CPU loop forward: h max abs err {_maxerr(h32, h_ref):.3g}, c {_maxerr(c32, c_ref):.3g}")
+    g32 = so.backward(*c.fwd_args(), c32, c.gh, c.gl, **kw32)
     _check_cells("grad_u", to_np(gu), g_ref[0], g32[0])
     _check_cells("grad_x", to_np(gx), g_ref[1], g32[1])
     _check_cells("grad_init", to_np(gi), g_ref[4], g32[4])
@@ -71,8 +75,11 @@ def test_headline_shape_against_float64_oracle(checkpointed):
     print(f"summed gradients vs float64: kernels grad_wc {e_wc:.3g} grad_bias {e_b:.3g}; "
           f"float32 CPU loop grad_wc {_maxerr(g32[2], g_ref[2]):.3g} grad_bias {_maxerr(g32[3], g_ref[3]):.3g}; "
           f"max|grad_wc| {np.abs(g_ref[2]).max():.3g} max|grad_bias| {np.abs(g_ref[3]).max():.3g}")
-    assert e_wc <= 1e-5 * max(1.0, np.abs(g_ref[2]).max())
-    assert e_b <= 1e-5 * max(1.0, np.abs(g_ref[3]).max())
+    # sums of 16 384 terms reaching magnitudes above 100 (one float32 ulp there is 7.6e-6): held to
+    # 1e-6 of the largest sum, ten times tighter than the per-cell rule, which is where the float32
+    # CPU loop lands as well
+    assert e_wc <= 1e-6 * max(1.0, np.abs(g_ref[2]).max())
+    assert e_b <= 1e-6 * max(1.0, np.abs(g_ref[3]).max())
 
 
 @pytest.mark.parametrize("checkpointed", [False, True], ids=["state_every_step", "state_checkpoints"])
