@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define SRU_AMD_ABI_VERSION 2
+#define SRU_AMD_ABI_VERSION 3
 
 enum sru_amd_dtype {
     SRU_AMD_F32 = 0,
@@ -59,7 +59,8 @@ enum sru_amd_status {
     SRU_AMD_ERR_BAD_DTYPE = 4,
     SRU_AMD_ERR_MISALIGNED = 5,     /* a stream pointer is not aligned to its element type */
     SRU_AMD_ERR_WORKSPACE = 6,      /* workspace missing or smaller than required */
-    SRU_AMD_ERR_LAUNCH = 7          /* the HIP runtime refused the launch */
+    SRU_AMD_ERR_LAUNCH = 7,         /* the HIP runtime refused the launch */
+    SRU_AMD_ERR_STATIC_LIMIT = 8    /* sru_amd_backward_static: more columns than its built-in scratch holds */
 };
 
 /* Problem description; the fields are the integer arguments of the reference's
@@ -135,6 +136,28 @@ int sru_amd_backward(const sru_amd_shape *shape,
                      void *grad_u, void *grad_x, void *grad_wc, float *grad_bias,
                      float *grad_init, void *workspace, size_t workspace_bytes,
                      void *stream);
+
+/* sru_amd_backward without the workspace argument, for callers that cannot allocate device
+ * memory at all: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc. It has no counterpart in the reference (whose operators allocate every output,
+ * sru/csrc/sru_cuda_impl.cpp:225-229). The per-column partial sums live in an array built into
+ * the library's device code (4 floats per column, 4 MiB, one copy per GPU for the life of the
+ * process), so the call allocates nothing and asks for nothing beyond inputs and outputs.
+ *   - at most SRU_AMD_STATIC_MAX_COLUMNS columns (B * D'); more returns
+ *     SRU_AMD_ERR_STATIC_LIMIT and launches nothing;
+ *   - results are bit-identical to sru_amd_backward's (same kernels);
+ *   - all calls on one GPU share that GPU's array: two calls that overlap in time on one GPU
+ *     (different streams, or two host threads) race; calls on one stream are safe back to back;
+ *   - the first call on a device resolves the array's address (hipGetSymbolAddress); make that
+ *     call outside a stream capture. */
+#define SRU_AMD_STATIC_MAX_COLUMNS 262144
+int sru_amd_backward_static(const sru_amd_shape *shape,
+                            const void *u, const void *x, const void *weight_c,
+                            const float *bias, const float *c_init, const float *mask_c,
+                            const uint8_t *mask_pad, const float *scale_x,
+                            const void *c, const void *grad_h, const float *grad_last,
+                            void *grad_u, void *grad_x, void *grad_wc, float *grad_bias,
+                            float *grad_init, void *stream);
 
 /* Static, NUL-terminated description of a status code (never NULL). The
  * reference has no counterpart: its operators throw (sru_cuda_impl_dummy.cpp:19)

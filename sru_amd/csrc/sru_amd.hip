@@ -8,9 +8,35 @@
 #include "sru_launch.h"
 #include "sru_reduce.h"
 
+#include <mutex>
+
 namespace {
 
 using namespace sru_amd;
+
+// Scratch of sru_amd_backward_static: the per-column partial sums (4 floats per column) of at most
+// SRU_AMD_STATIC_MAX_COLUMNS columns. One copy of the array exists on every device the library runs
+// on, at that device's own address, for the life of the process. In host code the array's name is
+// only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) float scratch[4 * SRU_AMD_STATIC_MAX_COLUMNS];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch`, per device ordinal
+
+// Address of the current device's copy of `scratch`; resolved once per device, on the first
+// call made with that device current. NULL if the runtime cannot tell.
+float *static_scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = static_cast<float *>(ptr);
+    }
+    return g_scratch_ptr[dev];
+}
 
 static_assert(SRU_AMD_STATE_INTERVAL == kCkptInterval, "header and kernels disagree");
 
@@ -49,7 +75,7 @@ int check_shape(const sru_amd_shape *s) {
     return SRU_AMD_OK;
 }
 
-// The backward call after the shape and workspace checks: pointer checks, then the
+// Everything sru_amd_backward and sru_amd_backward_static share: pointer checks, then the
 // scan and the batch reduction enqueued on `stream`, with the per-column partial sums in
 // `partial` (4 * B * D' floats of device memory).
 int backward_core(const sru_amd_shape *shape, const void *u, const void *x, const void *weight_c,
@@ -107,6 +133,8 @@ const char *sru_amd_status_string(int status) {
     case SRU_AMD_ERR_MISALIGNED: return "a stream pointer is not aligned to its element group";
     case SRU_AMD_ERR_WORKSPACE: return "workspace is NULL, misaligned or too small";
     case SRU_AMD_ERR_LAUNCH: return "the HIP runtime refused the kernel launch";
+    case SRU_AMD_ERR_STATIC_LIMIT:
+        return "more than SRU_AMD_STATIC_MAX_COLUMNS (262144) columns: use sru_amd_backward with a workspace";
     default: return "unknown status";
     }
 }
@@ -170,6 +198,19 @@ int sru_amd_backward(const sru_amd_shape *shape, const void *u, const void *x, c
         return SRU_AMD_ERR_WORKSPACE;
     return backward_core(shape, u, x, weight_c, bias, c_init, mask_c, mask_pad, scale_x, c, grad_h, grad_last,
                          grad_u, grad_x, grad_wc, grad_bias, grad_init, static_cast<float *>(workspace), stream);
+}
+
+int sru_amd_backward_static(const sru_amd_shape *shape, const void *u, const void *x, const void *weight_c,
+                            const float *bias, const float *c_init, const float *mask_c,
+                            const uint8_t *mask_pad, const float *scale_x, const void *c,
+                            const void *grad_h, const float *grad_last, void *grad_u, void *grad_x,
+                            void *grad_wc, float *grad_bias, float *grad_init, void *stream) {
+    if (const int rc = check_shape(shape)) return rc;
+    if (shape->batch * shape->hidden * shape->dirs > SRU_AMD_STATIC_MAX_COLUMNS) return SRU_AMD_ERR_STATIC_LIMIT;
+    float *partial = static_scratch_of_current_device();
+    if (!partial) return SRU_AMD_ERR_LAUNCH;
+    return backward_core(shape, u, x, weight_c, bias, c_init, mask_c, mask_pad, scale_x, c, grad_h, grad_last,
+                         grad_u, grad_x, grad_wc, grad_bias, grad_init, partial, stream);
 }
 
 }  // extern "C"

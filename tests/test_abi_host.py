@@ -85,6 +85,15 @@ def test_null_and_misaligned_pointers_and_workspace():
     assert lib.sru_amd_backward(ctypes.byref(s), *bad, need, None) == 1
 
 
+def test_static_backward_checks_sizes_before_anything_else():
+    # the allocation-free entry point refuses more columns than its built-in array holds
+    lib = _lib.load()
+    wide = _shape(batch=_lib.STATIC_MAX_COLUMNS // 16 + 1)
+    assert lib.sru_amd_backward_static(ctypes.byref(wide), *([FAKE] * 16), None) == 8
+    assert lib.sru_amd_backward_static(ctypes.byref(_shape(k=5)), *([FAKE] * 16), None) == 3
+    assert lib.sru_amd_backward_static(None, *([FAKE] * 16), None) == 1
+
+
 def test_status_strings_and_python_error_mapping():
     for code in range(0, 9):
         assert _lib.status_string(code)
