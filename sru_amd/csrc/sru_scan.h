@@ -274,17 +274,29 @@ struct Stream {
 #ifndef SRU_AMD_REFINE_SIGMOID
 #define SRU_AMD_REFINE_SIGMOID 1
 #endif
+constexpr float kNegLog2e = -1.4426950408889634f;
+
+// 1 / (1 + 2^t): the sigmoid of v for t = -log2(e) * v
 template <typename T>
-__device__ __forceinline__ float sigmoid(float v) {
+__device__ __forceinline__ float sigmoid_exp2(float t) {
     if constexpr (sizeof(T) == 4 && SRU_AMD_REFINE_SIGMOID) {
         // the exponent is capped so that d stays finite (inf * 0 in the correction would be NaN);
         // at the cap the result is 2^-126
-        const float d = 1.0f + __builtin_amdgcn_exp2f(fminf(-1.4426950408889634f * v, 126.0f));
+        const float d = 1.0f + __builtin_amdgcn_exp2f(fminf(t, 126.0f));
         const float r = __builtin_amdgcn_rcpf(d);
         return __builtin_fmaf(__builtin_fmaf(-d, r, 1.0f), r, r);
     } else {
-        return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v));
+        return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
     }
+}
+
+// A gate: sigmoid(u + w * c + b). The factor -log2(e) that turns exp into the hardware's exp2 is
+// folded into the operands: -log2(e) * w and -log2(e) * b are loop invariants (per-column constants,
+// hoisted by the compiler), and u enters through a multiply-add that does not wait for the state,
+// so the chain that does depend on the state c is one multiply-add, exp2, add, reciprocal.
+template <typename T>
+__device__ __forceinline__ float gate(float u, float w, float c, float b) {
+    return sigmoid_exp2<T>(__builtin_fmaf(kNegLog2e * w, c, __builtin_fmaf(kNegLog2e, u, kNegLog2e * b)));
 }
 
 // tanh through the same two units: 1 - 2 / (1 + e^(2v)). Absolute error below 3e-7 over the
@@ -441,8 +453,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
             const float u0 = s.u.get(c * K), u1 = s.u.get(c * K + 1), u2 = s.u.get(c * K + 2);
             const float w1 = custom ? s.w.get(2 * c) : wc1[c];
             const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
-            const float g1 = sigmoid<T>(u1 + w1 * cur[c] + b1[c]);
-            const float g2 = sigmoid<T>(u2 + w2 * cur[c] + b2[c]);
+            const float g1 = gate<T>(u1, w1, cur[c], b1[c]);
+            const float g2 = gate<T>(u2, w2, cur[c], b2[c]);
             const float cn = (cur[c] - u0) * g1 + u0;
             const float val = use_tanh ? tanh_fast(cn) : cn;
             float out;
@@ -590,8 +602,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float u0 = uu[c * K];
-                    const float g1 = sigmoid<T>(uu[c * K + 1] + wc1[c] * cur[c] + b1[c]);
-                    const float g2 = sigmoid<T>(uu[c * K + 2] + wc2[c] * cur[c] + b2[c]);
+                    const float g1 = gate<T>(uu[c * K + 1], wc1[c], cur[c], b1[c]);
+                    const float g2 = gate<T>(uu[c * K + 2], wc2[c], cur[c], b2[c]);
                     const float cn = (cur[c] - u0) * g1 + u0;
                     const float val = TANH ? tanh_fast(cn) : cn;
                     float out;
@@ -765,8 +777,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
             const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
             const float cp = s.first ? c_init[c] : s.cprev.get(c);
             const float u0 = s.u.get(c * K);
-            const float g1 = sigmoid<T>(s.u.get(c * K + 1) + w1 * cp + b1[c]);
-            const float g2 = sigmoid<T>(s.u.get(c * K + 2) + w2 * cp + b2[c]);
+            const float g1 = gate<T>(s.u.get(c * K + 1), w1, cp, b1[c]);
+            const float g2 = gate<T>(s.u.get(c * K + 2), w2, cp, b2[c]);
             const float val = use_tanh ? tanh_fast(cv[c]) : cv[c];
             const float dact = use_tanh ? (1.0f - val * val) : 1.0f;
             const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
@@ -944,8 +956,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                     const float cp = st[i][c];
                     u0s[i][c] = uu[c * K];
                     if (SKIP == 2) xs[i][c] = uu[c * K + K - 1];
-                    g1[i][c] = sigmoid<T>(uu[c * K + 1] + wc1[c] * cp + b1[c]);
-                    g2[i][c] = sigmoid<T>(uu[c * K + 2] + wc2[c] * cp + b2[c]);
+                    g1[i][c] = gate<T>(uu[c * K + 1], wc1[c], cp, b1[c]);
+                    g2[i][c] = gate<T>(uu[c * K + 2], wc2[c], cp, b2[c]);
                     const float cn = (cp - u0s[i][c]) * g1[i][c] + u0s[i][c];
                     st[i + 1][c] = padded ? cp : cn;
                 }
