@@ -149,6 +149,9 @@ def run_stack(args):
     import torch
     import sru_amd
     name, kw, L, B, n_in = STACKS[args.workload]
+    if args.torch_layer_norm:   # comparison run: torch's layer norm (and autocast's casts around it)
+        import sru_amd.modules
+        sru_amd.modules.fused_layer_norm_supported = lambda x: False
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
     model = sru_amd.SRU(**kw).to(dev)
@@ -201,7 +204,8 @@ def run_stack(args):
         "dtype": args.dtype if amp is None else args.dtype + " autocast", "data": "synthetic",
         "config": {"workload": name, "length": L, "batch": B, "layers": kw["num_layers"],
                    "pass": "forward only" if forward_only else "forward+backward",
-                   "replayed_from_graph": bool(args.graph)}}), flush=True)
+                   "replayed_from_graph": bool(args.graph),
+                   "layer_norm": "torch" if args.torch_layer_norm else "sru_amd kernels"}}), flush=True)
 
 
 def main():
@@ -223,6 +227,8 @@ def main():
                     help="side measurement: activation_type = tanh (the reference's deprecated use_tanh)")
     ap.add_argument("--graph", action="store_true",
                     help="with --workload stack1: record the forward into a HIP graph and time replays")
+    ap.add_argument("--torch-layer-norm", action="store_true",
+                    help="with a stack workload: use torch.nn.LayerNorm's kernels instead of this package's")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "

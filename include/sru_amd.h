@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define SRU_AMD_ABI_VERSION 3
+#define SRU_AMD_ABI_VERSION 4
 
 enum sru_amd_dtype {
     SRU_AMD_F32 = 0,
@@ -158,6 +158,33 @@ int sru_amd_backward_static(const sru_amd_shape *shape,
                             const void *c, const void *grad_h, const float *grad_last,
                             void *grad_u, void *grad_x, void *grad_wc, float *grad_bias,
                             float *grad_init, void *stream);
+
+/* Layer normalisation of the rows of a (rows, cols) matrix, the operation the reference applies to a
+ * layer's input before the projection or to its output after the recurrence with
+ * torch.nn.LayerNorm (sru/modules.py:155-162 created, :250-253 and :278-279 applied):
+ *   y = (x - mean(x)) / sqrt(var(x) + eps) * weight + bias,   statistics per row, biased variance.
+ * x and y may have different element types (enum sru_amd_dtype): the row is read once as it is
+ * and written in the type its consumer wants, which under autocast replaces a chain of three
+ * kernels (cast to float, normalise, cast to 16 bits). weight, bias, mean, rstd are float;
+ * mean and rstd (one value per row) are what the backward call needs.
+ *   cols must be a multiple of 8 and at most SRU_AMD_NORM_MAX_FEATURES; x, y, weight, bias
+ *   16-byte aligned. */
+#define SRU_AMD_NORM_MAX_FEATURES 4096
+int sru_amd_layer_norm_forward(int64_t rows, int64_t cols, const void *x, int x_dtype,
+                               const float *weight, const float *bias, float eps,
+                               void *y, int y_dtype, float *mean, float *rstd, void *stream);
+
+/* Bytes of device scratch sru_amd_layer_norm_backward needs (0 on a bad shape). */
+size_t sru_amd_layer_norm_backward_workspace_bytes(int64_t rows, int64_t cols);
+
+/* Backward of the above: grad_x (in x's element type) from grad_y (in y's element type), and the
+ * weight / bias gradients summed over rows in a fixed order (bit-reproducible). grad_weight and
+ * grad_bias must be the two halves of one (2, cols) float array: grad_bias == grad_weight + cols. */
+int sru_amd_layer_norm_backward(int64_t rows, int64_t cols, const void *x, int x_dtype,
+                                const float *weight, const float *mean, const float *rstd,
+                                const void *grad_y, int y_dtype, void *grad_x,
+                                float *grad_weight, float *grad_bias,
+                                void *workspace, size_t workspace_bytes, void *stream);
 
 /* Static, NUL-terminated description of a status code (never NULL). The
  * reference has no counterpart: its operators throw (sru_cuda_impl_dummy.cpp:19)

@@ -10,9 +10,10 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # SRU_AMD_LIBRARY points at another build of the same library (tuning builds)
 LIB_PATH = os.environ.get("SRU_AMD_LIBRARY") or os.path.join(_HERE, "libsru_amd.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 STATE_INTERVAL = 8   # SRU_AMD_STATE_INTERVAL
 STATIC_MAX_COLUMNS = 262144   # SRU_AMD_STATIC_MAX_COLUMNS
+NORM_MAX_FEATURES = 4096       # SRU_AMD_NORM_MAX_FEATURES
 
 F32, F16, BF16 = 0, 1, 2
 
@@ -41,6 +42,11 @@ SIGNATURES = {
     "sru_amd_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(Shape)]),
     "sru_amd_backward": (ctypes.c_int, [ctypes.POINTER(Shape)] + [_P] * 17 + [ctypes.c_size_t, _P]),
     "sru_amd_backward_static": (ctypes.c_int, [ctypes.POINTER(Shape)] + [_P] * 17),
+    "sru_amd_layer_norm_forward": (ctypes.c_int, [ctypes.c_int64, ctypes.c_int64, _P, ctypes.c_int, _P, _P,
+                                                  ctypes.c_float, _P, ctypes.c_int, _P, _P, _P]),
+    "sru_amd_layer_norm_backward_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int64, ctypes.c_int64]),
+    "sru_amd_layer_norm_backward": (ctypes.c_int, [ctypes.c_int64, ctypes.c_int64, _P, ctypes.c_int, _P, _P, _P, _P,
+                                                   ctypes.c_int, _P, _P, _P, _P, ctypes.c_size_t, _P]),
     "sru_amd_status_string": (ctypes.c_char_p, [ctypes.c_int]),
     "sru_amd_abi_version": (ctypes.c_int, []),
 }

@@ -290,13 +290,17 @@ __device__ __forceinline__ float sigmoid_exp2(float t) {
     }
 }
 
-// A gate: sigmoid(u + w * c + b). The factor -log2(e) that turns exp into the hardware's exp2 is
-// folded into the operands: -log2(e) * w and -log2(e) * b are loop invariants (per-column constants,
-// hoisted by the compiler), and u enters through a multiply-add that does not wait for the state,
-// so the chain that does depend on the state c is one multiply-add, exp2, add, reciprocal.
+// A gate: sigmoid(u + w * c + b). For 16-bit streams the factor -log2(e) that turns exp into the
+// hardware's exp2 is folded into the operands: -log2(e) * w and -log2(e) * b are loop invariants
+// (per-column constants, hoisted by the compiler), and u enters through a multiply-add that does
+// not wait for the state, so the chain that depends on the state c is one multiply-add, exp2,
+// add, reciprocal. Float streams keep the sum in its own scale and multiply afterwards: the folded
+// form rounds relative to the terms instead of to their (often much smaller) sum, which doubled the
+// largest gradient error at the headline shape.
 template <typename T>
 __device__ __forceinline__ float gate(float u, float w, float c, float b) {
-    return sigmoid_exp2<T>(__builtin_fmaf(kNegLog2e * w, c, __builtin_fmaf(kNegLog2e, u, kNegLog2e * b)));
+    if constexpr (sizeof(T) == 4) return sigmoid_exp2<T>(kNegLog2e * (u + w * c + b));
+    else return sigmoid_exp2<T>(__builtin_fmaf(kNegLog2e * w, c, __builtin_fmaf(kNegLog2e, u, kNegLog2e * b)));
 }
 
 // tanh through the same two units: 1 - 2 / (1 + e^(2v)). Absolute error below 3e-7 over the

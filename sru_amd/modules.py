@@ -18,6 +18,7 @@ import torch.nn as nn
 from torch import Tensor
 from torch.nn.utils.rnn import PackedSequence, pad_packed_sequence, pack_padded_sequence
 
+from .norm import layer_norm as fused_layer_norm, supported as fused_layer_norm_supported
 from .ops import elementwise_recurrence_gpu
 
 
@@ -131,7 +132,7 @@ class SRUCell(nn.Module):
 
         residual = input                                   # the skip term is the un-normalised input
         if self.layer_norm is not None and not self.normalize_after:
-            input = self.layer_norm(input)
+            input = self._normalise(input, feeds_projection=True)
         if self.training and self.rnn_dropout > 0:
             input = input * self._dropout_mask((batch, input.size(-1)), self.rnn_dropout)
         mask_c = None
@@ -142,8 +143,21 @@ class SRUCell(nn.Module):
         U, V = self.compute_UV(input, c0, mask_pad)
         h, c = self.apply_recurrence(U, V, residual, c0, scale_val, mask_c, mask_pad)
         if self.layer_norm is not None and self.normalize_after:
-            h = self.layer_norm(h)
+            h = self._normalise(h, feeds_projection=False)
         return h, c
+
+    def _normalise(self, x: Tensor, feeds_projection: bool) -> Tensor:
+        """self.layer_norm(x) (sru/modules.py:250-253, :278-279) through the layer-norm kernels of
+        this package where they apply. Before the projection under autocast the rows leave the
+        kernel in the autocast dtype, i.e. as the operand the dense product would otherwise obtain
+        by casting a float32 result; everywhere else the output keeps x's dtype."""
+        ln = self.layer_norm
+        if not fused_layer_norm_supported(x) or ln.weight is None or ln.bias is None:
+            return ln(x)
+        out_dtype = x.dtype
+        if feeds_projection and torch.is_autocast_enabled("cuda"):
+            out_dtype = torch.get_autocast_dtype("cuda")
+        return fused_layer_norm(x, ln.weight, ln.bias, ln.eps, out_dtype)
 
     def apply_recurrence(self, U: Tensor, V: Tensor, residual: Tensor, c0: Tensor,
                          scale_val: Optional[Tensor], mask_c: Optional[Tensor],

@@ -1,0 +1,78 @@
+"""Layer normalisation next to the recurrence (sru/modules.py:155-162, :250-253, :278-279).
+
+`layer_norm(x, weight, bias, eps, out_dtype)` is torch.nn.functional.layer_norm over the last
+dimension with one difference: the output dtype can be chosen, so that under autocast the
+normalised rows leave the kernel already in the 16-bit dtype the projection consumes. It runs the
+HIP kernels of csrc/sru_norm.hip through the C ABI (include/sru_amd.h); `supported()` says whether
+a tensor can take that path (device tensor, feature count a multiple of 8 and at most
+SRU_AMD_NORM_MAX_FEATURES) - anything else is torch's own layer_norm, which is the operation the
+reference itself calls.
+"""
+import ctypes
+from typing import Optional
+
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from . import _lib
+from .functional import _DTYPES, _aligned, _f32, _ptr
+
+
+def supported(x: Tensor) -> bool:
+    d = x.size(-1)
+    return bool(x.is_cuda and x.dtype in _DTYPES and x.numel() > 0 and d % 8 == 0 and d <= _lib.NORM_MAX_FEATURES)
+
+
+class LayerNormFunction(Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps, out_dtype):
+        D = x.size(-1)
+        x_ = _aligned(x, 16)
+        w_, b_ = _aligned(_f32(weight), 16), _aligned(_f32(bias), 16)
+        rows = x_.numel() // D
+        y = torch.empty(x_.shape, dtype=out_dtype, device=x.device)
+        mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+        with torch.cuda.device(x.device):
+            stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+            rc = _lib.load().sru_amd_layer_norm_forward(rows, D, _ptr(x_), _DTYPES[x_.dtype], _ptr(w_), _ptr(b_),
+                                                        ctypes.c_float(eps), _ptr(y), _DTYPES[out_dtype],
+                                                        _ptr(mean), _ptr(rstd), stream)
+        _lib.check(rc, "sru_amd_layer_norm_forward")
+        ctx.save_for_backward(x_, w_, mean, rstd)
+        ctx.param_dtypes = (weight.dtype, bias.dtype)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_y):
+        x_, w_, mean, rstd = ctx.saved_tensors
+        D = x_.size(-1)
+        rows = x_.numel() // D
+        gy = _aligned(grad_y, 16)
+        grad_x = torch.empty_like(x_)
+        grad_wb = torch.empty(2, D, dtype=torch.float32, device=x_.device)
+        lib = _lib.load()
+        nbytes = lib.sru_amd_layer_norm_backward_workspace_bytes(rows, D)
+        workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x_.device)
+        with torch.cuda.device(x_.device):
+            stream = ctypes.c_void_p(torch.cuda.current_stream(x_.device).cuda_stream)
+            rc = lib.sru_amd_layer_norm_backward(rows, D, _ptr(x_), _DTYPES[x_.dtype], _ptr(w_), _ptr(mean),
+                                                 _ptr(rstd), _ptr(gy), _DTYPES[gy.dtype], _ptr(grad_x),
+                                                 _ptr(grad_wb[0]), _ptr(grad_wb[1]), _ptr(workspace),
+                                                 ctypes.c_size_t(nbytes), stream)
+        _lib.check(rc, "sru_amd_layer_norm_backward")
+        wdt, bdt = ctx.param_dtypes
+        return grad_x, grad_wb[0].to(wdt), grad_wb[1].to(bdt), None, None
+
+
+def layer_norm(x: Tensor, weight: Tensor, bias: Tensor, eps: float = 1e-5,
+               out_dtype: Optional[torch.dtype] = None) -> Tensor:
+    """Normalises over the last dimension; `out_dtype` defaults to x's dtype."""
+    out_dtype = out_dtype or x.dtype
+    if out_dtype not in _DTYPES:
+        raise ValueError(f"out_dtype must be float32, float16 or bfloat16, not {out_dtype}")
+    if not supported(x):
+        y = torch.nn.functional.layer_norm(x.float(), (x.size(-1),), weight.float(), bias.float(), eps)
+        return y.to(out_dtype)
+    return LayerNormFunction.apply(x, weight, bias, eps, out_dtype)

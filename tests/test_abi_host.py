@@ -94,6 +94,27 @@ def test_static_backward_checks_sizes_before_anything_else():
     assert lib.sru_amd_backward_static(None, *([FAKE] * 16), None) == 1
 
 
+def test_layer_norm_entry_points_validate_before_launching():
+    lib = _lib.load()
+    f32 = 0
+    fwd = lambda rows, cols, x=FAKE, dx=f32, dy=f32: lib.sru_amd_layer_norm_forward(
+        rows, cols, x, dx, FAKE, FAKE, ctypes.c_float(1e-5), FAKE, dy, FAKE, FAKE, None)
+    assert fwd(0, 64) == 2 and fwd(4, 0) == 2 and fwd(4, 12) == 2          # cols must be a multiple of 8
+    assert fwd(4, _lib.NORM_MAX_FEATURES + 8) == 2
+    assert fwd(4, 64, dx=9) == 4 and fwd(4, 64, dy=5) == 4
+    assert fwd(4, 64, x=None) == 1
+    assert fwd(4, 64, x=ctypes.c_void_p(0x1004)) == 5
+    need = lib.sru_amd_layer_norm_backward_workspace_bytes(4, 64)
+    assert need == 1 * 2 * 64 * 4 and lib.sru_amd_layer_norm_backward_workspace_bytes(4, 12) == 0
+    assert lib.sru_amd_layer_norm_backward_workspace_bytes(10 ** 6, 1024) == 1024 * 2 * 1024 * 4
+    gw = ctypes.c_void_p(0x2000)
+    gb = ctypes.c_void_p(0x2000 + 64 * 4)
+    bwd = lambda ws, nbytes, gbias=gb: lib.sru_amd_layer_norm_backward(
+        4, 64, FAKE, f32, FAKE, FAKE, FAKE, FAKE, f32, FAKE, gw, gbias, ws, nbytes, None)
+    assert bwd(None, need) == 6 and bwd(FAKE, need - 1) == 6
+    assert bwd(FAKE, need, gbias=ctypes.c_void_p(0x3000)) == 5          # the two sums must be adjacent
+
+
 def test_status_strings_and_python_error_mapping():
     for code in range(0, 9):
         assert _lib.status_string(code)
