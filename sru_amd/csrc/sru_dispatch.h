@@ -13,7 +13,7 @@
 #include <cstdlib>
 
 #include "sru_launch.h"
-#include "sru_rows.h"
+#include "sru_split.h"
 
 namespace sru_amd {
 
@@ -30,21 +30,13 @@ constexpr int kNt = kNtLoad | kNtStore;
 // 1024 wavefronts) the kernels keep one column per lane and pair lanes for memory access.
 constexpr int64_t kPairBelow = 65536;
 
-// Row-tile kernels (sru_rows.h): 16-bit streams, every wavefront inside one direction and one
-// batch row, all streams 16-byte aligned, state kept as checkpoints or not at all.
-#ifndef SRU_AMD_ROWS_NBUF
-#define SRU_AMD_ROWS_NBUF 4   // chunks in flight per wavefront
-#endif
-constexpr int kRowsNbuf = SRU_AMD_ROWS_NBUF;
-// SRU_AMD_ROWS in the environment: 0 never, 2 wherever eligible, anything else the default rule
-// (a measurement knob; read once)
-inline int rows_policy() {
-    static const int v = [] { const char *e = std::getenv("SRU_AMD_ROWS"); return e ? std::atoi(e) : 1; }();
-    return v;
-}
-inline bool rows_wanted(int64_t ncols) {
-    const int policy = rows_policy();
-    return policy == 2 || (policy != 0 && ncols / 2 < kPairBelow);
+// Lane-pair kernels (sru_split.h): 16-bit streams, d a multiple of 32, at most 1024 wavefronts of 32
+// columns, every stream 16-byte aligned, state kept as checkpoints or not at all.
+constexpr int kSplitNbuf = 2;   // chunks (of 16 steps) in flight per wavefront
+// SRU_AMD_SPLIT=0 in the environment keeps them out (the one measurement knob; read once)
+inline bool split_wanted(int64_t ncols, int32_t d) {
+    static const bool enabled = [] { const char *e = std::getenv("SRU_AMD_SPLIT"); return !e || std::atoi(e) != 0; }();
+    return enabled && d % kSplitCols == 0 && ncols / kSplitCols <= 1024;
 }
 
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
@@ -117,26 +109,26 @@ hipError_t fast_backward(const BwdParams &p, hipStream_t st) {
 }
 
 template <typename T, int K, int SKIP, int X = 0, int STAGE = 0>
-hipError_t rows_forward(const FwdParams &p, hipStream_t st) {
+hipError_t split_forward(const FwdParams &p, hipStream_t st) {
     if constexpr (STAGE == 0) {
-        return p.act ? rows_forward<T, K, SKIP, X | kTanh, 1>(p, st) : rows_forward<T, K, SKIP, X, 1>(p, st);
+        return p.act ? split_forward<T, K, SKIP, X | kTanh, 1>(p, st) : split_forward<T, K, SKIP, X, 1>(p, st);
     } else if constexpr (STAGE == 1) {
-        return p.pad ? rows_forward<T, K, SKIP, X | kHasPad, 2>(p, st) : rows_forward<T, K, SKIP, X, 2>(p, st);
+        return p.pad ? split_forward<T, K, SKIP, X | kHasPad, 2>(p, st) : split_forward<T, K, SKIP, X, 2>(p, st);
     } else {
-        const dim3 grid = grid_for(p.ncols, 1);
-        if (p.ckpt) return launch(forward_scan_rows<T, K, SKIP, X | kNt | kCkpt, kCkptInterval, kRowsNbuf>, grid, st, p);
-        return launch(forward_scan_rows<T, K, SKIP, X | kNt, kCkptInterval, kRowsNbuf>, grid, st, p);
+        const dim3 grid((unsigned)(p.ncols / kSplitCols));
+        if (p.ckpt) return launch(forward_scan_split<T, K, SKIP, X | kNt | kCkpt, kSplitNbuf>, grid, st, p);
+        return launch(forward_scan_split<T, K, SKIP, X | kNt, kSplitNbuf>, grid, st, p);
     }
 }
 
 template <typename T, int K, int SKIP, int X = 0, int STAGE = 0>
-hipError_t rows_backward(const BwdParams &p, hipStream_t st) {
+hipError_t split_backward(const BwdParams &p, hipStream_t st) {
     if constexpr (STAGE == 0) {
-        return p.act ? rows_backward<T, K, SKIP, X | kTanh, 1>(p, st) : rows_backward<T, K, SKIP, X, 1>(p, st);
+        return p.act ? split_backward<T, K, SKIP, X | kTanh, 1>(p, st) : split_backward<T, K, SKIP, X, 1>(p, st);
     } else {
-        const dim3 grid = grid_for(p.ncols, 1);
-        if (p.pad) return launch(backward_scan_rows<T, K, SKIP, X | kNt | kHasPad, kCkptInterval, kRowsNbuf>, grid, st, p);
-        return launch(backward_scan_rows<T, K, SKIP, X | kNt, kCkptInterval, kRowsNbuf>, grid, st, p);
+        const dim3 grid((unsigned)(p.ncols / kSplitCols));
+        if (p.pad) return launch(backward_scan_split<T, K, SKIP, X | kNt | kHasPad, kSplitNbuf>, grid, st, p);
+        return launch(backward_scan_split<T, K, SKIP, X | kNt, kSplitNbuf>, grid, st, p);
     }
 }
 
@@ -149,8 +141,8 @@ inline bool all_aligned_16(std::initializer_list<const void *> ptrs) {
 template <typename T, int K, int SKIP>
 hipError_t pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
-        if (!p.c && wave_uniform(p.d, 1) && rows_wanted(p.ncols) && all_aligned_16({p.u, p.x, p.h}))
-            return rows_forward<T, K, SKIP>(p, st);
+        if (!p.c && split_wanted(p.ncols, p.d) && all_aligned_16({p.u, p.x, p.h}))
+            return split_forward<T, K, SKIP>(p, st);
     }
     if constexpr (Tune<T>::kCols == 2) {
         if (pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c})) {
@@ -164,8 +156,8 @@ hipError_t pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t 
 template <typename T, int K, int SKIP>
 hipError_t pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
-        if (p.ckpt && wave_uniform(p.d, 1) && rows_wanted(p.ncols) && all_aligned_16({p.u, p.x, p.gh, p.gu, p.gx}))
-            return rows_backward<T, K, SKIP>(p, st);
+        if (p.ckpt && split_wanted(p.ncols, p.d) && all_aligned_16({p.u, p.x, p.gh, p.gu, p.gx}))
+            return split_backward<T, K, SKIP>(p, st);
     }
     if constexpr (Tune<T>::kCols == 2) {
         if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) {  // p.c is null with checkpoints
