@@ -227,6 +227,9 @@ def main():
                     help="side measurement: activation_type = tanh (the reference's deprecated use_tanh)")
     ap.add_argument("--graph", action="store_true",
                     help="with --workload stack1: record the forward into a HIP graph and time replays")
+    ap.add_argument("--per-step-weight-c", action="store_true",
+                    help="side measurement: weight_c given per step, (L, B, D', 2) in the stream dtype (the "
+                         "reference's custom_m returning V)")
     ap.add_argument("--torch-layer-norm", action="store_true",
                     help="with a stack workload: use torch.nn.LayerNorm's kernels instead of this package's")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -257,14 +260,17 @@ def main():
     tdt = TORCH_DT[args.dtype]
     es = DT_BYTES[args.dtype]
     lib = _lib.load()
-    ckpt = not args.full_state and not fwd_only and not (args.no_skip and k == 4)
+    custom = args.per_step_weight_c
+    ckpt = not args.full_state and not fwd_only and not (args.no_skip and k == 4) and not (custom and args.tanh)
     use_x = k == 3 and not args.no_skip      # the skip term is read from x
     if args.tanh:
         name += " tanh"
     if args.no_skip:
         name += " no skip term"
+    if custom:
+        name += " per-step weight_c"
     shape = _lib.Shape(L, B, d, dirs, k, 1 if args.tanh else 0,
-                       0 if args.no_skip else (1 if k == 3 else 2), 0, CODE[args.dtype],
+                       0 if args.no_skip else (1 if k == 3 else 2), 1 if custom else 0, CODE[args.dtype],
                        _lib.STATE_INTERVAL if ckpt else 1)
     state_rows = lib.sru_amd_state_bytes(ctypes.byref(shape)) // (B * Dp * (4 if ckpt else DT_BYTES[args.dtype]))
 
@@ -282,6 +288,8 @@ def main():
         )
         sets.append(s)
     wc = (torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1) * 1.5 ** 0.5
+    if custom:
+        wc = (wc.view(2, Dp).t().reshape(1, 1, 2 * Dp) + 0.1 * torch.randn(L, B, 2 * Dp, device=dev, generator=g)).to(tdt)
     bias = torch.zeros(2 * Dp, device=dev)
     c0 = torch.zeros(B, Dp, device=dev)
     gl = torch.zeros(B, Dp, device=dev)
@@ -291,7 +299,7 @@ def main():
     if padded:
         lens = torch.randint(L // 4, L + 1, (B,), device=dev, generator=g)
         pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :]).view(torch.uint8).contiguous()
-    gwc = torch.empty(2 * Dp, device=dev)
+    gwc = torch.empty(L, B, 2 * Dp, device=dev, dtype=tdt) if custom else torch.empty(2 * Dp, device=dev)
     gb = torch.empty(2 * Dp, device=dev)
     gi = torch.empty(B, Dp, device=dev)
     ws_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(shape))
@@ -359,7 +367,8 @@ def main():
     # sessions on this same command; the file is named in the output
     traffic, traffic_source = None, None
     tfile = os.path.join(ROOT, "profiles", "traffic_bi_d1024_L256_B64_%s.json" % args.dtype)
-    if args.workload == "headline" and ckpt and not args.tanh and not args.no_skip and os.path.exists(tfile):
+    if args.workload == "headline" and ckpt and not args.tanh and not args.no_skip and not custom \
+            and os.path.exists(tfile):
         rec = json.load(open(tfile))
         traffic = rec["backward_scan"]["traffic_bytes"]
         traffic_source = ("replayed from profiles/%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, %s); "
@@ -367,13 +376,15 @@ def main():
     # Reference algorithm (what `achieved` and `frac` are priced on): forward reads U (k) and x (k=3
     # with a skip term), writes h and (training) the state c after every step; backward reads U (k),
     # x, c, grad_h and writes grad_u (k), grad_x.
-    fwd_bytes = (k + (1 if use_x else 0) + (1 if fwd_only else 2)) * es * cells
-    bwd_bytes = (2 * k + (2 if use_x else 0) + 2) * es * cells
+    # (a per-step weight_c is one more stream of 2 elements per cell: read by both passes, its
+    # gradient written by the backward pass)
+    fwd_bytes = (k + (1 if use_x else 0) + (1 if fwd_only else 2) + (2 if custom else 0)) * es * cells
+    bwd_bytes = (2 * k + (2 if use_x else 0) + 2 + (4 if custom else 0)) * es * cells
     # What the selected kernels are built to move: with checkpoints the per-step state (es bytes per
     # cell each way) shrinks to one float per 8 steps.
     state_bytes = (4 * cells // 8) if ckpt else es * cells
-    fwd_moved = (k + (1 if use_x else 0) + 1) * es * cells + (0 if fwd_only else state_bytes)
-    bwd_moved = (2 * k + (2 if use_x else 0) + 1) * es * cells + state_bytes
+    fwd_moved = (k + (1 if use_x else 0) + 1 + (2 if custom else 0)) * es * cells + (0 if fwd_only else state_bytes)
+    bwd_moved = (2 * k + (2 if use_x else 0) + 1 + (4 if custom else 0)) * es * cells + state_bytes
     if fwd_only:
         bwd_us = float("nan")
     bwd_gbs = bwd_bytes / (bwd_us * 1e-6) / 1e9

@@ -60,10 +60,13 @@ int check_shape(const sru_amd_shape *s) {
         return SRU_AMD_ERR_BAD_DTYPE;
     if (s->state_interval != 0 && s->state_interval != 1 && s->state_interval != SRU_AMD_STATE_INTERVAL)
         return SRU_AMD_ERR_BAD_FLAGS;
-    // checkpointed state exists only for the fast kernels
-    if (s->state_interval == SRU_AMD_STATE_INTERVAL &&
-        (s->is_custom != 0 || (s->skip_type == 0 && s->k == 4)))
-        return SRU_AMD_ERR_BAD_FLAGS;
+    // checkpointed state exists only for the chunked kernels: not for four streams without a skip
+    // term; with a per-step weight_c not together with tanh, and 16-bit streams then need an even d
+    if (s->state_interval == SRU_AMD_STATE_INTERVAL) {
+        if (s->skip_type == 0 && s->k == 4) return SRU_AMD_ERR_BAD_FLAGS;
+        if (s->is_custom != 0 && (s->activation_type != 0 || (s->dtype != SRU_AMD_F32 && s->hidden % 2 != 0)))
+            return SRU_AMD_ERR_BAD_FLAGS;
+    }
     // D' must fit an int, the grid must fit 2^31-1 workgroups and the largest stream
     // (L*B*D'*k elements) must stay far inside the 64-bit byte offsets the kernels use.
     const int64_t lim = INT64_C(1) << 31;
@@ -96,6 +99,11 @@ int backward_core(const sru_amd_shape *shape, const void *u, const void *x, cons
         !aligned(weight_c, s.is_custom ? 2 * es : 4) || !aligned(grad_wc, s.is_custom ? 2 * es : 4) ||
         !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(grad_last, 4) || !aligned(grad_bias, 4) ||
         !aligned(grad_init, 4) || (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
+        return SRU_AMD_ERR_MISALIGNED;
+
+    if (ckpt && s.is_custom && es == 2 &&
+        (!aligned(u, s.k == 4 ? 16 : 4) || !aligned(grad_u, s.k == 4 ? 16 : 4) || !aligned(weight_c, 8) ||
+         !aligned(grad_wc, 8) || !aligned(grad_h, 4) || (s.skip_type == 1 && (!aligned(x, 4) || !aligned(grad_x, 4)))))
         return SRU_AMD_ERR_MISALIGNED;
 
     BwdParams p{};
@@ -154,6 +162,11 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
         (s.skip_type == 1 && !aligned(x, es)) || !aligned(weight_c, s.is_custom ? 2 * es : 4) ||
         !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(c_last, 4) ||
         (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
+        return SRU_AMD_ERR_MISALIGNED;
+
+    // a per-step weight_c with checkpoints and 16-bit streams moves two columns per lane
+    if (ckpt && s.is_custom && es == 2 &&
+        (!aligned(u, s.k == 4 ? 16 : 4) || !aligned(weight_c, 8) || !aligned(h, 4) || (s.skip_type == 1 && !aligned(x, 4))))
         return SRU_AMD_ERR_MISALIGNED;
 
     FwdParams p{};

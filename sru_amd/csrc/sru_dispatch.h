@@ -73,7 +73,9 @@ inline bool wave_uniform(int32_t d, int cols) { return d % (kBlock * cols) == 0;
 // properties are turned into template bits one at a time.
 template <typename T, int K, int SKIP, int COLS, int X = 0, int STAGE = 0>
 hipError_t fast_forward(const FwdParams &p, hipStream_t st) {
-    if constexpr (STAGE == 0) {
+    if constexpr (STAGE == 0 && (X & kCustom) != 0) {   // (a per-step weight_c with tanh runs the general kernels)
+        return fast_forward<T, K, SKIP, COLS, X, 1>(p, st);
+    } else if constexpr (STAGE == 0) {
         return p.act ? fast_forward<T, K, SKIP, COLS, X | kTanh, 1>(p, st) : fast_forward<T, K, SKIP, COLS, X, 1>(p, st);
     } else if constexpr (STAGE == 1) {
         return wave_uniform(p.d, COLS) ? fast_forward<T, K, SKIP, COLS, X | kUniform, 2>(p, st)
@@ -85,20 +87,24 @@ hipError_t fast_forward(const FwdParams &p, hipStream_t st) {
         const dim3 grid = grid_for(p.ncols, COLS);
         // what is kept for the backward pass: checkpoints, the state after every step, or nothing
         if (p.ckpt) return launch(forward_scan_chunked<T, K, SKIP, X | kNt | kCkpt, COLS, TC>, grid, st, p);
-        if (p.c) return launch(forward_scan_chunked<T, K, SKIP, X | kNt | kKeepC, COLS, TC>, grid, st, p);
+        if constexpr ((X & kCustom) == 0) {   // (with a per-step weight_c the state after every step is the general kernels')
+            if (p.c) return launch(forward_scan_chunked<T, K, SKIP, X | kNt | kKeepC, COLS, TC>, grid, st, p);
+        }
         return launch(forward_scan_chunked<T, K, SKIP, X | kNt, COLS, TC>, grid, st, p);
     }
 }
 
 template <typename T, int K, int SKIP, int COLS, int X = 0, int STAGE = 0>
 hipError_t fast_backward(const BwdParams &p, hipStream_t st) {
-    if constexpr (STAGE == 0) {
+    if constexpr (STAGE == 0 && (X & kCustom) != 0) {
+        return fast_backward<T, K, SKIP, COLS, X, 1>(p, st);
+    } else if constexpr (STAGE == 0) {
         return p.act ? fast_backward<T, K, SKIP, COLS, X | kTanh, 1>(p, st) : fast_backward<T, K, SKIP, COLS, X, 1>(p, st);
     } else if constexpr (STAGE == 1) {
         return p.pad ? fast_backward<T, K, SKIP, COLS, X | kHasPad, 2>(p, st) : fast_backward<T, K, SKIP, COLS, X, 2>(p, st);
     } else {
         const dim3 grid = grid_for(p.ncols, COLS);
-        if constexpr ((X & kPair) == 0) {   // (lane pairing exists in the chunked kernels only)
+        if constexpr ((X & (kPair | kCustom)) == 0) {   // (lane pairing and the weight_c stream exist in the chunked kernels only)
             // reference-style state: the ring kernel reads it step by step
             if (!p.ckpt) return launch(backward_scan<T, K, SKIP, X | kNt, COLS, kRingDepth>, grid, st, p);
         }
@@ -169,8 +175,36 @@ hipError_t pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t
 }
 
 // (k, skip_type) pairs that pass the shape check: (3,0) (3,1) (4,0) (4,2).
+// A per-step weight_c runs the chunked kernels (with the weight_c stream compiled in) when the
+// activation is the identity, the state is kept as checkpoints or not at all, and, for 16-bit
+// streams, columns can be paired; everything else about it is the general kernels' business.
+template <typename T, int K>
+bool custom_chunked_ok(const sru_amd_shape &s, bool full_state, std::initializer_list<const void *> wide,
+                       std::initializer_list<const void *> mid, std::initializer_list<const void *> narrow) {
+    if (!s.is_custom || s.activation_type != 0 || full_state || (s.skip_type == 0 && s.k == 4)) return false;
+    if (sizeof(T) == 4) return true;
+    for (const void *q : mid)
+        if (q && !aligned_to(q, 8)) return false;
+    return pair_ok<T, K>(s, wide, narrow);
+}
+
+template <typename T, int K, int SKIP>
+hipError_t custom_forward(const FwdParams &p, hipStream_t st) {
+    return fast_forward<T, K, SKIP, Tune<T>::kCols, kCustom>(p, st);
+}
+template <typename T, int K, int SKIP>
+hipError_t custom_backward(const BwdParams &p, hipStream_t st) {
+    return fast_backward<T, K, SKIP, Tune<T>::kCols, kCustom>(p, st);
+}
+
 template <typename T>
 hipError_t launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
+    if (s.k == 3 ? custom_chunked_ok<T, 3>(s, p.c != nullptr, {p.u}, {p.wc}, {p.x, p.h})
+                 : custom_chunked_ok<T, 4>(s, p.c != nullptr, {p.u}, {p.wc}, {p.x, p.h})) {
+        if (s.k == 4) return custom_forward<T, 4, 2>(p, st);
+        if (s.skip_type == 1) return custom_forward<T, 3, 1>(p, st);
+        return custom_forward<T, 3, 0>(p, st);
+    }
     const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
     if (!general) {
         if (s.k == 4) return pick_forward<T, 4, 2>(s, p, st);
@@ -187,6 +221,13 @@ hipError_t launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_
 
 template <typename T>
 hipError_t launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
+    if (s.k == 3 ? custom_chunked_ok<T, 3>(s, p.ckpt == nullptr, {p.u, p.gu}, {p.wc, p.gwc_steps}, {p.x, p.gh, p.gx})
+                 : custom_chunked_ok<T, 4>(s, p.ckpt == nullptr, {p.u, p.gu}, {p.wc, p.gwc_steps}, {p.x, p.gh, p.gx})) {
+        if (s.k == 4) return custom_backward<T, 4, 2>(p, st);
+        if (s.skip_type == 1) return custom_backward<T, 3, 1>(p, st);
+        return custom_backward<T, 3, 0>(p, st);
+    }
+    if (s.is_custom && p.ckpt) return hipErrorInvalidValue;   // (refused by the shape and alignment checks before)
     const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
     if (!general) {
         if (s.k == 4) return pick_backward<T, 4, 2>(s, p, st);

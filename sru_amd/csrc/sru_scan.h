@@ -354,6 +354,7 @@ constexpr int kNtStore = 16; // MODE bit: stream stores are non-temporal
 constexpr int kCkpt = 32;    // MODE bit (fast forward kernels): store a state checkpoint per chunk
 constexpr int kPair = 64;    // MODE bit (chunked fast kernels, 16-bit): lanes pair up for memory access
 constexpr int kTanh = 256;   // MODE bit (fast kernels): the output uses tanh(c_t) instead of c_t
+constexpr int kCustom = 512; // MODE bit (chunked fast kernels): weight_c is a stream, (L, B, D', 2) in T
 constexpr int kUniform = 128;// MODE bit (chunked fast kernels): a wavefront lies inside one direction and
                              // one batch row (d is a multiple of 64 * COLS), so the time index, the row
                              // pointers and the padding flag are scalar: no per-lane address arithmetic
@@ -524,7 +525,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
     constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
-    constexpr bool TANH = (MODE & kTanh) != 0;
+    constexpr bool TANH = (MODE & kTanh) != 0, CUSTOM = (MODE & kCustom) != 0;
     // Wave-uniform kernels with a padding mask: all lanes of a wavefront share the flags, so one
     // load per chunk fetches them (lane l the flag of step l % TC) instead of one load per step,
     // which leaves more of the 64 outstanding memory operations a wavefront may have to the
@@ -534,6 +535,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
+    using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c: two elements per column
     const uint32_t wg = blockIdx.x;
     const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
@@ -551,8 +553,8 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], cur[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        wc1[c] = static_cast<const float *>(p.wc)[j + c];
-        wc2[c] = static_cast<const float *>(p.wc)[Dp + j + c];
+        wc1[c] = CUSTOM ? 0.f : static_cast<const float *>(p.wc)[j + c];
+        wc2[c] = CUSTOM ? 0.f : static_cast<const float *>(p.wc)[Dp + j + c];
         b1[c] = p.bias[j + c];
         b2[c] = p.bias[Dp + j + c];
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
@@ -571,10 +573,12 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     const T *xbase = static_cast<const T *>(p.x);
     T *hbase = static_cast<T *>(p.h);
     T *cbase = static_cast<T *>(p.c);
+    const T *vbase = static_cast<const T *>(p.wc);   // CUSTOM only
 
     struct Chunk {
         typename SU::G u[TC];
         typename S1::G x[TC];
+        typename SV::G w[CUSTOM ? TC : 1];
         uint32_t pad[kPadRegs];  // padding flags of the chunk, see load_chunk
     };
 
@@ -586,6 +590,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
                 const int64_t e = ef + (s0 + i) * es;
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
                 if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
+                if constexpr (CUSTOM) k.w[i] = SV::template load<NTL>(vbase + e * 2, lane, q);
                 if (!PAD_BY_LANE) k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
@@ -603,11 +608,13 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
                 float hv[COLS], cv[COLS], uu[COLS * K], xx[COLS] = {};
                 SU::unpack(k.u[i], q, uu);
                 if (SKIP == 1) S1::unpack(k.x[i], q, xx);
+                float ww[COLS * 2] = {};
+                if constexpr (CUSTOM) SV::unpack(k.w[i], q, ww);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float u0 = uu[c * K];
-                    const float g1 = gate<T>(uu[c * K + 1], wc1[c], cur[c], b1[c]);
-                    const float g2 = gate<T>(uu[c * K + 2], wc2[c], cur[c], b2[c]);
+                    const float g1 = gate<T>(uu[c * K + 1], CUSTOM ? ww[2 * c] : wc1[c], cur[c], b1[c]);
+                    const float g2 = gate<T>(uu[c * K + 2], CUSTOM ? ww[2 * c + 1] : wc2[c], cur[c], b2[c]);
                     const float cn = (cur[c] - u0) * g1 + u0;
                     const float val = TANH ? tanh_fast(cn) : cn;
                     float out;
@@ -871,9 +878,10 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
     // (forward_scan_chunked fetches the flags of a chunk with one load; here, where every flag
     // is needed twice, that measured 0-3 % slower, so the flags stay one load per step)
-    constexpr bool TANH = (MODE & kTanh) != 0;
+    constexpr bool TANH = (MODE & kTanh) != 0, CUSTOM = (MODE & kCustom) != 0;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
+    using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c and its gradient: two elements per column
     const uint32_t wg = blockIdx.x;
     const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
@@ -891,8 +899,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     CompensatedSum sw1[COLS], sw2[COLS], sb1[COLS], sb2[COLS];  // weight_c / bias gradient sums over the walk
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        wc1[c] = static_cast<const float *>(p.wc)[j + c];
-        wc2[c] = static_cast<const float *>(p.wc)[Dp + j + c];
+        wc1[c] = CUSTOM ? 0.f : static_cast<const float *>(p.wc)[j + c];
+        wc2[c] = CUSTOM ? 0.f : static_cast<const float *>(p.wc)[Dp + j + c];
         b1[c] = p.bias[j + c];
         b2[c] = p.bias[Dp + j + c];
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
@@ -914,11 +922,14 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     const T *ghbase = static_cast<const T *>(p.gh);
     T *gubase = static_cast<T *>(p.gu);
     T *gxbase = static_cast<T *>(p.gx);
+    const T *vbase = static_cast<const T *>(p.wc);   // CUSTOM only
+    T *gvbase = static_cast<T *>(p.gwc_steps);
 
     struct Chunk {
         typename SU::G u[TC];
         typename S1::G x[TC];
         typename S1::G gh[TC];
+        typename SV::G w[CUSTOM ? TC : 1];
         uint32_t pad[TC];    // padding flags of the chunk's steps
         float cstart[COLS];  // state before the chunk's first step
     };
@@ -933,6 +944,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
                 if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
                 k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
+                if constexpr (CUSTOM) k.w[i] = SV::template load<NTL>(vbase + e * 2, lane, q);
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
@@ -955,13 +967,15 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 const bool padded = k.pad[i] != 0;
                 float uu[COLS * K];
                 SU::unpack(k.u[i], q, uu);
+                float ww[COLS * 2] = {};
+                if constexpr (CUSTOM) SV::unpack(k.w[i], q, ww);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float cp = st[i][c];
                     u0s[i][c] = uu[c * K];
                     if (SKIP == 2) xs[i][c] = uu[c * K + K - 1];
-                    g1[i][c] = gate<T>(uu[c * K + 1], wc1[c], cp, b1[c]);
-                    g2[i][c] = gate<T>(uu[c * K + 2], wc2[c], cp, b2[c]);
+                    g1[i][c] = gate<T>(uu[c * K + 1], CUSTOM ? ww[2 * c] : wc1[c], cp, b1[c]);
+                    g2[i][c] = gate<T>(uu[c * K + 2], CUSTOM ? ww[2 * c + 1] : wc2[c], cp, b2[c]);
                     const float cn = (cp - u0s[i][c]) * g1[i][c] + u0s[i][c];
                     st[i + 1][c] = padded ? cp : cn;
                 }
@@ -974,6 +988,8 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 float gu[COLS * K], gx[COLS], xx[COLS] = {}, ghs[COLS];
                 if (SKIP == 1) S1::unpack(k.x[i], q, xx);
                 S1::unpack(k.gh[i], q, ghs);
+                float ww[COLS * 2] = {}, gv[COLS * 2];
+                if constexpr (CUSTOM) SV::unpack(k.w[i], q, ww);
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) {
                     const float cp = st[i][c];
@@ -988,7 +1004,9 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                     const float gc = TANH ? gh * m[c] * (G2 * dact) + cur[c] : gh * m[c] * G2 + cur[c];
                     const float gg1 = gc * (cp - u0) * (G1 * (1.0f - G1));
                     const float gskip = gh * (1.0f - G2 * m[c]);
-                    const float ncur = gc * G1 + gg1 * wc1[c] + gg2 * wc2[c];
+                    const float ncur = gc * G1 + gg1 * (CUSTOM ? ww[2 * c] : wc1[c]) + gg2 * (CUSTOM ? ww[2 * c + 1] : wc2[c]);
+                    gv[2 * c] = padded ? 0.0f : gg1 * cp;
+                    gv[2 * c + 1] = padded ? 0.0f : gg2 * cp;
 
                     gu[c * K] = padded ? 0.0f : gc * (1.0f - G1);
                     gu[c * K + 1] = padded ? 0.0f : gg1;
@@ -1004,6 +1022,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
                 const int64_t e = ef + (s0 + i) * es;
                 SU::template store<NTS>(gubase + e * K, lane, q, gu);
                 if (SKIP == 1) S1::template store<NTS>(gxbase + e, lane, q, gx);
+                if constexpr (CUSTOM) SV::template store<NTS>(gvbase + e * 2, lane, q, gv);
             }
         }
 #pragma unroll

@@ -76,10 +76,11 @@ class _Problem:
         self.dtype = u.dtype
         self.squeeze = x.dim() == 2
         # Between forward and backward keep float checkpoints of the state instead of the
-        # state after every step wherever the kernels support it (no per-step weight_c; with
-        # four streams, a skip term): the backward kernel rebuilds what lies in between.
-        self.checkpointed = bool(checkpoint_state and not self.is_custom
-                                 and not (self.skip_type == 0 and self.k == 4))
+        # state after every step wherever the kernels support it (with four streams, a skip
+        # term): the backward kernel rebuilds what lies in between.
+        # With a per-step weight_c: not together with tanh, and 16-bit streams need an even d.
+        custom_ok = not self.is_custom or (activation_type == 0 and (u.dtype == torch.float32 or d_out % 2 == 0))
+        self.checkpointed = bool(checkpoint_state and custom_ok and not (self.skip_type == 0 and self.k == 4))
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
                                 activation_type, self.skip_type, self.is_custom,
                                 _DTYPES[u.dtype],
@@ -91,7 +92,7 @@ class _Problem:
 
 
 def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad):
-    u_ = _aligned(u, pb.group_bytes())
+    u_ = _aligned(u, max(4, pb.group_bytes()))
     x_ = None
     if pb.skip_type == 1:
         x_ = _aligned(x if x.dtype == pb.dtype else x.to(pb.dtype), 4)

@@ -125,7 +125,14 @@ def test_mid_shapes(cfg, dt):
     check_against_oracle(Case(seed=22, **cfg), dt)
 
 
-FAST = [g for g in GRID + MID if not g.get("custom") and (g.get("skip", True) or g.get("k", 3) == 3)]
+# every layout that can keep its state as checkpoints: all but four streams without a skip term and
+# a per-step weight_c together with tanh
+FAST = [g for g in GRID + MID if (g.get("skip", True) or g.get("k", 3) == 3)
+        and not (g.get("custom") and g.get("act"))]
+FAST += [dict(L=21, B=3, d=64, dirs=2, custom=True, k=4, pad="right"),
+         dict(L=33, B=2, d=70, custom=True, pad="random", mask_c=True, scale=1.3),
+         dict(L=17, B=4, d=128, dirs=2, custom=True, skip=False),
+         dict(L=40, B=2, d=192, custom=True, scale=0.7)]
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
@@ -206,14 +213,19 @@ def test_padded_cells_cannot_leak_bit_identical():
     assert float(out_a[4][pad].abs().max()) == 0.0      # grad_x
 
 
-def test_backward_is_bit_reproducible():
-    c = Case(L=50, B=16, d=256, dirs=2, seed=35, pad="right")
-    a = DeviceProblem(c)
-    a.forward()
-    first = [t.clone() for t in a.backward()]
-    for _ in range(3):
-        again = a.backward()
-        assert all(torch.equal(p, q) for p, q in zip(first, again))
+@pytest.mark.parametrize("dt,checkpointed", [("f32", False), ("f32", True), ("bf16", True), ("f16", True)])
+def test_backward_is_bit_reproducible(dt, checkpointed):
+    # also: repeated backward calls on one state buffer (the checkpoint kernels count arrivals in
+    # it to add up the batch sums and must leave the counters as they found them)
+    for cfg in (dict(L=50, B=16, d=256, dirs=2, pad="right"), dict(L=23, B=5, d=96, dirs=1, k=4),
+                dict(L=9, B=1, d=64, dirs=2, mask_c=True)):
+        c = Case(seed=35, **cfg)
+        a = DeviceProblem(c, dt, checkpointed=checkpointed)
+        a.forward()
+        first = [None if t is None else t.clone() for t in a.backward()]
+        for _ in range(3):
+            again = a.backward()
+            assert all(p is None or torch.equal(p, q) for p, q in zip(first, again))
 
 
 def _random_cases(n, seed):
@@ -244,7 +256,7 @@ def _random_cases(n, seed):
                                        int(os.environ.get("SRU_AMD_RANDOM_SEED", "2024"))),
                          ids=lambda v: _ids(v) if isinstance(v, dict) else str(v))
 def test_random_draws_over_shapes_and_flags(cfg, dt, checkpointed, seed):
-    fast = not cfg["custom"] and (cfg["skip"] or cfg["k"] == 3)
+    fast = (cfg["skip"] or cfg["k"] == 3) and not (cfg["custom"] and (cfg["act"] or (dt != "f32" and cfg["d"] % 2)))
     check_against_oracle(Case(seed=seed, **cfg), dt, checkpointed=checkpointed and fast)
 
 
