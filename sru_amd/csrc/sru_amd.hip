@@ -61,11 +61,12 @@ int check_shape(const sru_amd_shape *s) {
     if (s->state_interval != 0 && s->state_interval != 1 && s->state_interval != SRU_AMD_STATE_INTERVAL)
         return SRU_AMD_ERR_BAD_FLAGS;
     // checkpointed state exists only for the chunked kernels: not for four streams without a skip
-    // term; with a per-step weight_c not together with tanh, and 16-bit streams then need an even d
+    // term, not for a per-step weight_c together with tanh, and 16-bit streams need an even d
+    // (their chunked kernels move two columns at a time)
     if (s->state_interval == SRU_AMD_STATE_INTERVAL) {
         if (s->skip_type == 0 && s->k == 4) return SRU_AMD_ERR_BAD_FLAGS;
-        if (s->is_custom != 0 && (s->activation_type != 0 || (s->dtype != SRU_AMD_F32 && s->hidden % 2 != 0)))
-            return SRU_AMD_ERR_BAD_FLAGS;
+        if (s->is_custom != 0 && s->activation_type != 0) return SRU_AMD_ERR_BAD_FLAGS;
+        if (s->dtype != SRU_AMD_F32 && s->hidden % 2 != 0) return SRU_AMD_ERR_BAD_FLAGS;
     }
     // D' must fit an int, the grid must fit 2^31-1 workgroups and the largest stream
     // (L*B*D'*k elements) must stay far inside the 64-bit byte offsets the kernels use.
@@ -101,9 +102,10 @@ int backward_core(const sru_amd_shape *shape, const void *u, const void *x, cons
         !aligned(grad_init, 4) || (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
         return SRU_AMD_ERR_MISALIGNED;
 
-    if (ckpt && s.is_custom && es == 2 &&
-        (!aligned(u, s.k == 4 ? 16 : 4) || !aligned(grad_u, s.k == 4 ? 16 : 4) || !aligned(weight_c, 8) ||
-         !aligned(grad_wc, 8) || !aligned(grad_h, 4) || (s.skip_type == 1 && (!aligned(x, 4) || !aligned(grad_x, 4)))))
+    if (ckpt && es == 2 &&
+        (!aligned(u, s.k == 4 ? 16 : 4) || !aligned(grad_u, s.k == 4 ? 16 : 4) ||
+         (s.is_custom && (!aligned(weight_c, 8) || !aligned(grad_wc, 8))) || !aligned(grad_h, 4) ||
+         (s.skip_type == 1 && (!aligned(x, 4) || !aligned(grad_x, 4)))))
         return SRU_AMD_ERR_MISALIGNED;
 
     BwdParams p{};
@@ -164,9 +166,10 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
         (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
         return SRU_AMD_ERR_MISALIGNED;
 
-    // a per-step weight_c with checkpoints and 16-bit streams moves two columns per lane
-    if (ckpt && s.is_custom && es == 2 &&
-        (!aligned(u, s.k == 4 ? 16 : 4) || !aligned(weight_c, 8) || !aligned(h, 4) || (s.skip_type == 1 && !aligned(x, 4))))
+    // 16-bit streams with checkpoints move two columns at a time
+    if (ckpt && es == 2 &&
+        (!aligned(u, s.k == 4 ? 16 : 4) || (s.is_custom && !aligned(weight_c, 8)) || !aligned(h, 4) ||
+         (s.skip_type == 1 && !aligned(x, 4))))
         return SRU_AMD_ERR_MISALIGNED;
 
     FwdParams p{};

@@ -145,18 +145,29 @@ inline bool all_aligned_16(std::initializer_list<const void *> ptrs) {
 }
 
 template <typename T, int K, int SKIP>
+hipError_t general_forward(const FwdParams &p, hipStream_t st) {
+    return launch(forward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, grid_for(p.ncols, 1), st, p);
+}
+template <typename T, int K, int SKIP>
+hipError_t general_backward(const BwdParams &p, hipStream_t st) {
+    return launch(backward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, grid_for(p.ncols, 1), st, p);
+}
+
+// 16-bit streams whose columns cannot be paired (odd d, or a stream pointer that is not aligned to a
+// pair's group) run the general kernels, one column per lane with 2-byte accesses; the host side
+// refuses checkpointed state for them.
+template <typename T, int K, int SKIP>
 hipError_t pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
         if (!p.c && split_wanted(p.ncols, p.d) && all_aligned_16({p.u, p.x, p.h}))
             return split_forward<T, K, SKIP>(p, st);
+        if (!pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c}))
+            return p.ckpt ? hipErrorInvalidValue : general_forward<T, K, SKIP>(p, st);
+        if (p.ncols / 2 < kPairBelow) return fast_forward<T, K, SKIP, 1, kPair>(p, st);
+        return fast_forward<T, K, SKIP, 2>(p, st);
+    } else {
+        return fast_forward<T, K, SKIP, 1>(p, st);
     }
-    if constexpr (Tune<T>::kCols == 2) {
-        if (pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c})) {
-            if (p.ncols / 2 < kPairBelow) return fast_forward<T, K, SKIP, 1, kPair>(p, st);
-            return fast_forward<T, K, SKIP, 2>(p, st);
-        }
-    }
-    return fast_forward<T, K, SKIP, 1>(p, st);
 }
 
 template <typename T, int K, int SKIP>
@@ -164,14 +175,13 @@ hipError_t pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t
     if constexpr (sizeof(T) == 2) {
         if (p.ckpt && split_wanted(p.ncols, p.d) && all_aligned_16({p.u, p.x, p.gh, p.gu, p.gx}))
             return split_backward<T, K, SKIP>(p, st);
+        if (!pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx}))   // p.c is null with checkpoints
+            return p.ckpt ? hipErrorInvalidValue : general_backward<T, K, SKIP>(p, st);
+        if (p.ckpt && p.ncols / 2 < kPairBelow) return fast_backward<T, K, SKIP, 1, kPair>(p, st);
+        return fast_backward<T, K, SKIP, 2>(p, st);
+    } else {
+        return fast_backward<T, K, SKIP, 1>(p, st);
     }
-    if constexpr (Tune<T>::kCols == 2) {
-        if (pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx})) {  // p.c is null with checkpoints
-            if (p.ckpt && p.ncols / 2 < kPairBelow) return fast_backward<T, K, SKIP, 1, kPair>(p, st);
-            return fast_backward<T, K, SKIP, 2>(p, st);
-        }
-    }
-    return fast_backward<T, K, SKIP, 1>(p, st);
 }
 
 // (k, skip_type) pairs that pass the shape check: (3,0) (3,1) (4,0) (4,2).
@@ -211,12 +221,10 @@ hipError_t launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_
         if (s.skip_type == 1) return pick_forward<T, 3, 1>(s, p, st);
         return pick_forward<T, 3, 0>(s, p, st);
     }
-    const dim3 grid = grid_for(p.ncols, 1);
-    constexpr int P = kRingDepth, M = kGeneral | kNt;
-    if (s.k == 3 && s.skip_type == 1) return launch(forward_scan<T, 3, 1, M, 1, P>, grid, st, p);
-    if (s.k == 3) return launch(forward_scan<T, 3, 0, M, 1, P>, grid, st, p);
-    if (s.skip_type == 2) return launch(forward_scan<T, 4, 2, M, 1, P>, grid, st, p);
-    return launch(forward_scan<T, 4, 0, M, 1, P>, grid, st, p);
+    if (s.k == 3 && s.skip_type == 1) return general_forward<T, 3, 1>(p, st);
+    if (s.k == 3) return general_forward<T, 3, 0>(p, st);
+    if (s.skip_type == 2) return general_forward<T, 4, 2>(p, st);
+    return general_forward<T, 4, 0>(p, st);
 }
 
 template <typename T>
@@ -234,12 +242,10 @@ hipError_t launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream
         if (s.skip_type == 1) return pick_backward<T, 3, 1>(s, p, st);
         return pick_backward<T, 3, 0>(s, p, st);
     }
-    const dim3 grid = grid_for(p.ncols, 1);
-    constexpr int P = kRingDepth, M = kGeneral | kNt;
-    if (s.k == 3 && s.skip_type == 1) return launch(backward_scan<T, 3, 1, M, 1, P>, grid, st, p);
-    if (s.k == 3) return launch(backward_scan<T, 3, 0, M, 1, P>, grid, st, p);
-    if (s.skip_type == 2) return launch(backward_scan<T, 4, 2, M, 1, P>, grid, st, p);
-    return launch(backward_scan<T, 4, 0, M, 1, P>, grid, st, p);
+    if (s.k == 3 && s.skip_type == 1) return general_backward<T, 3, 1>(p, st);
+    if (s.k == 3) return general_backward<T, 3, 0>(p, st);
+    if (s.skip_type == 2) return general_backward<T, 4, 2>(p, st);
+    return general_backward<T, 4, 0>(p, st);
 }
 
 }  // namespace sru_amd

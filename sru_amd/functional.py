@@ -78,9 +78,9 @@ class _Problem:
         # Between forward and backward keep float checkpoints of the state instead of the
         # state after every step wherever the kernels support it (with four streams, a skip
         # term): the backward kernel rebuilds what lies in between.
-        # With a per-step weight_c: not together with tanh, and 16-bit streams need an even d.
-        custom_ok = not self.is_custom or (activation_type == 0 and (u.dtype == torch.float32 or d_out % 2 == 0))
-        self.checkpointed = bool(checkpoint_state and custom_ok and not (self.skip_type == 0 and self.k == 4))
+        # 16-bit streams need an even d for that; a per-step weight_c must not come with tanh.
+        ok = (u.dtype == torch.float32 or d_out % 2 == 0) and not (self.is_custom and activation_type != 0)
+        self.checkpointed = bool(checkpoint_state and ok and not (self.skip_type == 0 and self.k == 4))
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
                                 activation_type, self.skip_type, self.is_custom,
                                 _DTYPES[u.dtype],

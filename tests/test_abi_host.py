@@ -45,7 +45,7 @@ FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
     (dict(skip_type=2, k=3), 3), (dict(is_custom=2), 3), (dict(dtype=7), 4),
     (dict(state_interval=4), 3),
     (dict(state_interval=8, is_custom=1, activation_type=1), 3), (dict(state_interval=8, skip_type=0, k=4), 3),
-    (dict(state_interval=8, is_custom=1, dtype=2, hidden=7), 3),
+    (dict(state_interval=8, dtype=2, hidden=7), 3), (dict(state_interval=8, dtype=1, hidden=1), 3),
 ])
 def test_forward_rejects_bad_shapes(kw, code):
     lib = _lib.load()
