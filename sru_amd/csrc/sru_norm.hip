@@ -5,13 +5,14 @@
 // the consumer wants (the 16-bit operand of the projection under autocast), which replaces the
 // chain "cast to float, normalise, cast to 16 bits" that autocast builds around torch's kernel.
 //
-// Mapping: one wavefront per row (a row = the D features of one (t, b) position); a lane holds
-// 8 consecutive features per pass of 512, so rows of float move as two 16-byte vectors per lane
-// and pass, 16-bit rows as one. Statistics are float: mean first, then the variance of the
-// centred values (both wavefront reductions). The backward kernel walks rows with a stride of the
-// grid's wavefront count, keeps its share of the weight / bias gradient sums in registers,
-// combines the block's wavefronts through LDS in a fixed order and leaves one partial row per
-// block; reduce_rows() then adds the blocks in index order, in double: bit-reproducible.
+// Mapping: one workgroup per row at a time (a row = the D features of one (t, b) position), 1 to 8
+// wavefronts of which every lane holds 8 consecutive features, so rows of float move as two
+// 16-byte vectors per lane, 16-bit rows as one; workgroups walk rows with a stride of the grid and
+// load the next row while they reduce the current one. Statistics are float: mean first, then the
+// variance of the centred values (wavefront reductions combined through LDS in wavefront order).
+// The backward kernel keeps each lane's share of the weight / bias gradient sums in registers over
+// the rows its workgroup visits and leaves one partial row per workgroup; reduce_rows() then adds
+// the workgroups in index order, in double: bit-reproducible.
 #include "sru_amd.h"
 
 #include <hip/hip_runtime.h>
@@ -25,7 +26,6 @@ using namespace sru_amd;
 constexpr int kLanes = 64;
 constexpr int kPer = 8;                       // features per lane and pass
 constexpr int kPass = kLanes * kPer;          // features per pass of a wavefront
-constexpr int kNormWaves = 4;                 // wavefronts (rows in flight) per workgroup
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -59,172 +59,261 @@ template <typename T> __device__ __forceinline__ void store8(T *p, const float (
     *reinterpret_cast<u32x4 *>(p) = a;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
+// A lane's 8 features of one row as they come from memory: loaded without a condition (the
+// callers clamp the address), so that the load can stay in flight across a loop trip, and turned
+// into floats only when the row's turn comes.
+template <typename T> struct Raw {
+    u32x4 a;
+    __device__ __forceinline__ void load(const T *p) { a = *reinterpret_cast<const u32x4 *>(p); }
+    __device__ __forceinline__ void unpack(float (&v)[kPer]) const {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kLanes);
-    return v;
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i] = bits_to_float<T>(a[i] & 0xffffu);
+            v[2 * i + 1] = bits_to_float<T>(a[i] >> 16);
+        }
+    }
+};
+template <> struct Raw<float> {
+    f32x4 a, b;
+    __device__ __forceinline__ void load(const float *p) {
+        a = *reinterpret_cast<const f32x4 *>(p);
+        b = *reinterpret_cast<const f32x4 *>(p + 4);
+    }
+    __device__ __forceinline__ void unpack(float (&v)[kPer]) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+    }
+};
+
+// v of another lane, chosen by a data-parallel-primitive control word; lanes outside row_mask get 0
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+
+// Sum over the wavefront, the same value in every lane: pairs, quads, then the four quads of each
+// row of 16 lanes by rotation, then row 0 into row 1 and row 2 into row 3, rows 0-1 into rows 2-3,
+// and the last lane's total to all.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp<0xB1>(v);         // quad_perm [1,0,3,2]
+    v += dpp<0x4E>(v);         // quad_perm [2,3,0,1]
+    v += dpp<0x124>(v);        // row_ror 4
+    v += dpp<0x128>(v);        // row_ror 8
+    v += dpp<0x142, 0xA>(v);   // row_bcast 15 into rows 1 and 3
+    v += dpp<0x143, 0xC>(v);   // row_bcast 31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+// Rows a workgroup handles per trip: their loads are in flight together and their sums share a barrier.
+constexpr int kRowsPer = 2;
+
+// Sums over the workgroup (the WAVES wavefronts that share a row) of N values at once, the
+// wavefronts' shares added in wavefront order. `red` holds N * WAVES floats and must not be
+// rewritten before every thread has read it (the callers alternate two arrays so that the next
+// barrier provides that).
+template <int WAVES, int N>
+__device__ __forceinline__ void block_sums(float (&v)[N], float *red) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) v[n] = wave_sum(v[n]);
+    if constexpr (WAVES > 1) {
+        if ((threadIdx.x & (kLanes - 1)) == 0) {
+#pragma unroll
+            for (int n = 0; n < N; ++n) red[n * WAVES + (threadIdx.x >> 6)] = v[n];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            v[n] = red[n * WAVES];
+#pragma unroll
+            for (int w = 1; w < WAVES; ++w) v[n] += red[n * WAVES + w];
+        }
+    }
 }
 
 // y = (x - mean) * rstd * gamma + beta per row; mean and rstd (float, one per row) are kept for
-// the backward pass. MAXP: passes of 512 features a lane can hold (D <= 512 * MAXP).
-template <typename TI, typename TO, int MAXP>
-__global__ void __launch_bounds__(kLanes * kNormWaves)
+// the backward pass. A workgroup of WAVES wavefronts owns kRowsPer consecutive rows at a time, every
+// lane 8 consecutive features of each (D <= 512 * WAVES), and walks the row groups with a stride of
+// the grid; the next group's loads are issued before the current group's reductions.
+template <typename TI, typename TO, int WAVES>
+__global__ void __launch_bounds__(kLanes * WAVES)
 layer_norm_forward(const TI *x, const float *gamma, const float *beta, TO *y, float *mean, float *rstd,
                    int64_t rows, int32_t D, float eps) {
-    const int lane = threadIdx.x & (kLanes - 1);
-    const int64_t first = (int64_t)blockIdx.x * kNormWaves + (threadIdx.x >> 6);
-    const int64_t stride = (int64_t)gridDim.x * kNormWaves;
-    float g[MAXP][kPer], b[MAXP][kPer];
-#pragma unroll
-    for (int p = 0; p < MAXP; ++p) {
-        const int e = p * kPass + lane * kPer;
-        if (e < D) {
-            load8<float>(gamma + e, g[p]);
-            load8<float>(beta + e, b[p]);
-        }
+    constexpr int R = kRowsPer;
+    __shared__ float red_a[R * WAVES], red_b[R * WAVES];
+    const int e = threadIdx.x * kPer;
+    const bool active = e < D;
+    float g[kPer] = {}, b[kPer] = {};
+    if (active) {
+        load8<float>(gamma + e, g);
+        load8<float>(beta + e, b);
     }
     const float inv_d = 1.0f / (float)D;
-    for (int64_t row = first; row < rows; row += stride) {
-        float v[MAXP][kPer];
-        float s = 0.f;
+    const TI *mine = x + (active ? e : 0);   // lanes past the row's end re-read its start and drop it
+    const int64_t last = rows - 1;
+    Raw<TI> next[R];
+    int64_t row = (int64_t)blockIdx.x * R;
 #pragma unroll
-        for (int p = 0; p < MAXP; ++p) {
-            const int e = p * kPass + lane * kPer;
-            if (e < D) {
-                load8<TI>(x + row * D + e, v[p]);
+    for (int r = 0; r < R; ++r) next[r].load(mine + (row + r < last ? row + r : last) * D);
+    for (; row < rows; row += (int64_t)gridDim.x * R) {
+        float v[R][kPer], s[R], q[R];
 #pragma unroll
-                for (int i = 0; i < kPer; ++i) s += v[p][i];
+        for (int r = 0; r < R; ++r) next[r].unpack(v[r]);
+        const int64_t after = row + (int64_t)gridDim.x * R;
+#pragma unroll
+        for (int r = 0; r < R; ++r) next[r].load(mine + (after + r < last ? after + r : last) * D);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            s[r] = 0.f;
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                v[r][i] = active ? v[r][i] : 0.f;
+                s[r] += v[r][i];
             }
         }
-        const float mu = wave_sum(s) * inv_d;
-        float q = 0.f;
+        block_sums<WAVES, R>(s, red_a);
 #pragma unroll
-        for (int p = 0; p < MAXP; ++p) {
-            if (p * kPass + lane * kPer < D) {
+        for (int r = 0; r < R; ++r) {
+            s[r] *= inv_d;
+            q[r] = 0.f;
+            if (active) {
 #pragma unroll
                 for (int i = 0; i < kPer; ++i) {
-                    v[p][i] -= mu;
-                    q += v[p][i] * v[p][i];
+                    v[r][i] -= s[r];
+                    q[r] += v[r][i] * v[r][i];
                 }
             }
         }
-        const float rs = 1.0f / sqrtf(wave_sum(q) * inv_d + eps);
+        block_sums<WAVES, R>(q, red_b);
 #pragma unroll
-        for (int p = 0; p < MAXP; ++p) {
-            const int e = p * kPass + lane * kPer;
-            if (e < D) {
+        for (int r = 0; r < R; ++r) {
+            if (row + r >= rows) break;
+            const float rs = rsqrtf(q[r] * inv_d + eps);
+            if (active) {
                 float o[kPer];
 #pragma unroll
-                for (int i = 0; i < kPer; ++i) o[i] = v[p][i] * rs * g[p][i] + b[p][i];
-                store8<TO>(y + row * D + e, o);
+                for (int i = 0; i < kPer; ++i) o[i] = v[r][i] * rs * g[i] + b[i];
+                store8<TO>(y + (row + r) * D + e, o);
             }
-        }
-        if (lane == 0) {
-            mean[row] = mu;
-            rstd[row] = rs;
+            if (threadIdx.x == 0) {
+                mean[row + r] = s[r];
+                rstd[row + r] = rs;
+            }
         }
     }
 }
 
 // dx = rstd * (g - mean(g) - xhat * mean(g * xhat)) with g = dy * gamma, xhat = (x - mean) * rstd;
-// partial[block] = (sum over the block's rows of dy * xhat, sum of dy), each D floats.
-template <typename TI, typename TG, typename TD, int MAXP>
-__global__ void __launch_bounds__(kLanes * kNormWaves)
+// partial[block] = (sum over the block's rows of dy * xhat, sum of dy), each D floats: every feature
+// belongs to one lane of the workgroup, which adds its rows in the order it visits them.
+template <typename TI, typename TG, typename TD, int WAVES>
+__global__ void __launch_bounds__(kLanes * WAVES)
 layer_norm_backward(const TI *x, const float *gamma, const float *mean, const float *rstd, const TG *dy, TD *dx,
                     float *partial, int64_t rows, int32_t D) {
-    extern __shared__ float acc[];   // (2, D): the block's sums
-    const int lane = threadIdx.x & (kLanes - 1);
-    const int wave = threadIdx.x >> 6;
-    const int64_t first = (int64_t)blockIdx.x * kNormWaves + wave;
-    const int64_t stride = (int64_t)gridDim.x * kNormWaves;
-    float g[MAXP][kPer], dg[MAXP][kPer], db[MAXP][kPer];
-#pragma unroll
-    for (int p = 0; p < MAXP; ++p) {
-        const int e = p * kPass + lane * kPer;
-        if (e < D) load8<float>(gamma + e, g[p]);
-#pragma unroll
-        for (int i = 0; i < kPer; ++i) dg[p][i] = db[p][i] = 0.f;
-    }
+    constexpr int R = kRowsPer;
+    __shared__ float red[2][2 * R * WAVES];   // alternate by trip: one barrier per trip
+    const int e = threadIdx.x * kPer;
+    const bool active = e < D;
+    float g[kPer] = {}, dg[kPer] = {}, db[kPer] = {};
+    if (active) load8<float>(gamma + e, g);
     const float inv_d = 1.0f / (float)D;
-    for (int64_t row = first; row < rows; row += stride) {
-        const float mu = mean[row], rs = rstd[row];
-        float xh[MAXP][kPer], gy[MAXP][kPer];
-        float s1 = 0.f, s2 = 0.f;
+    const int ec = active ? e : 0;   // lanes past the row's end re-read its start and drop it
+    const TI *my_x = x + ec;
+    const TG *my_dy = dy + ec;
+    const int64_t last = rows - 1;
+    Raw<TI> nx[R];
+    Raw<TG> nd[R];
+    int64_t row = (int64_t)blockIdx.x * R;
 #pragma unroll
-        for (int p = 0; p < MAXP; ++p) {
-            const int e = p * kPass + lane * kPer;
-            if (e < D) {
-                float d[kPer];
-                load8<TI>(x + row * D + e, xh[p]);
-                load8<TG>(dy + row * D + e, d);
+    for (int r = 0; r < R; ++r) {
+        const int64_t at = (row + r < last ? row + r : last) * D;
+        nx[r].load(my_x + at);
+        nd[r].load(my_dy + at);
+    }
+    int parity = 0;
+    for (; row < rows; row += (int64_t)gridDim.x * R, parity ^= 1) {
+        float xh[R][kPer], gy[R][kPer], sums[2 * R], rs[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            nx[r].unpack(xh[r]);
+            nd[r].unpack(gy[r]);
+        }
+        const int64_t after = row + (int64_t)gridDim.x * R;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t at = (after + r < last ? after + r : last) * D;
+            nx[r].load(my_x + at);
+            nd[r].load(my_dy + at);
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const bool live = row + r < rows;   // a row past the end repeats the last row and is dropped
+            const float mu = live ? mean[row + r] : 0.f;
+            rs[r] = live ? rstd[row + r] : 0.f;
+            float s1 = 0.f, s2 = 0.f;
+            if (live) {
 #pragma unroll
                 for (int i = 0; i < kPer; ++i) {
-                    xh[p][i] = (xh[p][i] - mu) * rs;
-                    gy[p][i] = d[i] * g[p][i];
-                    s1 += gy[p][i];
-                    s2 += gy[p][i] * xh[p][i];
-                    dg[p][i] += d[i] * xh[p][i];
-                    db[p][i] += d[i];
+                    const float d = active ? gy[r][i] : 0.f;
+                    xh[r][i] = (xh[r][i] - mu) * rs[r];
+                    gy[r][i] = d * g[i];
+                    s1 += gy[r][i];
+                    s2 += gy[r][i] * xh[r][i];
+                    dg[i] += d * xh[r][i];
+                    db[i] += d;
                 }
             }
+            sums[2 * r] = s1;
+            sums[2 * r + 1] = s2;
         }
-        const float c1 = wave_sum(s1) * inv_d, c2 = wave_sum(s2) * inv_d;
+        block_sums<WAVES, 2 * R>(sums, red[parity]);
 #pragma unroll
-        for (int p = 0; p < MAXP; ++p) {
-            const int e = p * kPass + lane * kPer;
-            if (e < D) {
-                float o[kPer];
+        for (int r = 0; r < R; ++r) {
+            if (row + r >= rows || !active) continue;
+            const float c1 = sums[2 * r] * inv_d, c2 = sums[2 * r + 1] * inv_d;
+            float o[kPer];
 #pragma unroll
-                for (int i = 0; i < kPer; ++i) o[i] = rs * (gy[p][i] - c1 - xh[p][i] * c2);
-                store8<TD>(dx + row * D + e, o);
-            }
+            for (int i = 0; i < kPer; ++i) o[i] = rs[r] * (gy[r][i] - c1 - xh[r][i] * c2);
+            store8<TD>(dx + (row + r) * D + e, o);
         }
     }
-    // the block's wavefronts add their sums one after the other: a fixed order
-    for (int w = 0; w < kNormWaves; ++w) {
-        if (wave == w) {
-#pragma unroll
-            for (int p = 0; p < MAXP; ++p) {
-                const int e = p * kPass + lane * kPer;
-                if (e < D) {
-#pragma unroll
-                    for (int i = 0; i < kPer; ++i) {
-                        acc[e + i] = (w == 0 ? 0.f : acc[e + i]) + dg[p][i];
-                        acc[D + e + i] = (w == 0 ? 0.f : acc[D + e + i]) + db[p][i];
-                    }
-                }
-            }
-        }
-        __syncthreads();
+    if (active) {
+        float *out = partial + (int64_t)blockIdx.x * 2 * D;
+        store8<float>(out + e, dg);
+        store8<float>(out + D + e, db);
     }
-    float *out = partial + (int64_t)blockIdx.x * 2 * D;
-    for (int e = threadIdx.x; e < 2 * D; e += blockDim.x) out[e] = acc[e];
 }
 
-// out[e] = sum over r of partial[r][e]. One workgroup per 64 columns; its 16 wavefronts take every
-// 16th row each, accumulate in double and are combined through LDS in a fixed order.
+// out[slab][e] = sum over the slab's rows r of partial[r][e]; slab = blockIdx.y takes rows
+// [slab * chunk, (slab + 1) * chunk). One workgroup per 64 columns and slab; its 16 wavefronts take
+// every 16th row each, accumulate in double and are combined through LDS in a fixed order. Many
+// rows go in two launches (float rows -> kSlabs double rows -> one float row), few in one.
 constexpr int kRowSlices = 16;
+constexpr int kSlabs = 16;
+template <typename TIN, typename TOUT>
 __global__ void __launch_bounds__(kLanes * kRowSlices)
-reduce_rows(const float *partial, float *out, int32_t nrows, int32_t width) {
+reduce_rows(const TIN *partial, TOUT *out, int32_t nrows, int32_t width, int32_t chunk) {
     __shared__ double part[kRowSlices][kLanes];
     const int lane = threadIdx.x & (kLanes - 1), slice = threadIdx.x >> 6;
     const int e = blockIdx.x * kLanes + lane;
+    const int first = blockIdx.y * chunk;
+    const int end = first + chunk < nrows ? first + chunk : nrows;
     double s = 0.0;
     if (e < width)
-        for (int r = slice; r < nrows; r += kRowSlices) s += (double)partial[(int64_t)r * width + e];
+        for (int r = first + slice; r < end; r += kRowSlices) s += (double)partial[(int64_t)r * width + e];
     part[slice][lane] = s;
     __syncthreads();
     if (slice == 0 && e < width) {
         double total = part[0][lane];
 #pragma unroll
         for (int i = 1; i < kRowSlices; ++i) total += part[i][lane];
-        out[e] = (float)total;
+        out[(int64_t)blockIdx.y * width + e] = (TOUT)total;
     }
 }
 
+// Workgroups of a launch: each walks groups of kRowsPer rows with a stride of the grid.
 int norm_blocks(int64_t rows) {
-    const int64_t want = (rows + kNormWaves - 1) / kNormWaves;
-    return (int)(want < 1024 ? want : 1024);   // 4096 wavefronts at most: 4 per SIMD
+    const int64_t groups = (rows + kRowsPer - 1) / kRowsPer;
+    return (int)(groups < 1024 ? groups : 1024);
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
@@ -237,19 +326,24 @@ int check_norm(int64_t rows, int64_t cols, int dt_a, int dt_b) {
     return SRU_AMD_OK;
 }
 
+// wavefronts per row: 8 features per lane
+inline int norm_waves(int32_t D) {
+    const int need = (D + kPass - 1) / kPass;
+    return need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
+}
+
 template <typename TI, typename TO>
 hipError_t launch_norm_forward(const void *x, const float *gamma, const float *beta, void *y, float *mean,
                                float *rstd, int64_t rows, int32_t D, float eps, hipStream_t st) {
     const TI *xi = static_cast<const TI *>(x);
     TO *yo = static_cast<TO *>(y);
     void *args[] = {&xi, &gamma, &beta, &yo, &mean, &rstd, &rows, &D, &eps};
-    const dim3 grid(norm_blocks(rows)), block(kLanes * kNormWaves);
-    const int passes = (D + kPass - 1) / kPass;
-    const void *k = passes <= 1   ? reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 1>)
-                    : passes <= 2 ? reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 2>)
-                    : passes <= 4 ? reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 4>)
-                                  : reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 8>);
-    return hipLaunchKernel(k, grid, block, args, 0, st);
+    const int waves = norm_waves(D);
+    const void *k = waves == 1   ? reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 1>)
+                    : waves == 2 ? reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 2>)
+                    : waves == 4 ? reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 4>)
+                                 : reinterpret_cast<const void *>(layer_norm_forward<TI, TO, 8>);
+    return hipLaunchKernel(k, dim3(norm_blocks(rows)), dim3(kLanes * waves), args, 0, st);
 }
 
 template <typename TI, typename TG, typename TD>
@@ -259,14 +353,12 @@ hipError_t launch_norm_backward(const void *x, const float *gamma, const float *
     const TG *gi = static_cast<const TG *>(dy);
     TD *di = static_cast<TD *>(dx);
     void *args[] = {&xi, &gamma, &mean, &rstd, &gi, &di, &partial, &rows, &D};
-    const dim3 grid(norm_blocks(rows)), block(kLanes * kNormWaves);
-    const size_t lds = (size_t)2 * D * sizeof(float);
-    const int passes = (D + kPass - 1) / kPass;
-    const void *k = passes <= 1   ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 1>)
-                    : passes <= 2 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 2>)
-                    : passes <= 4 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 4>)
-                                  : reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 8>);
-    return hipLaunchKernel(k, grid, block, args, lds, st);
+    const int waves = norm_waves(D);
+    const void *k = waves == 1   ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 1>)
+                    : waves == 2 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 2>)
+                    : waves == 4 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 4>)
+                                 : reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 8>);
+    return hipLaunchKernel(k, dim3(norm_blocks(rows)), dim3(kLanes * waves), args, 0, st);
 }
 
 // run F<A, B>(...) for the two runtime dtypes
@@ -308,7 +400,8 @@ int sru_amd_layer_norm_forward(int64_t rows, int64_t cols, const void *x, int x_
 
 size_t sru_amd_layer_norm_backward_workspace_bytes(int64_t rows, int64_t cols) {
     if (check_norm(rows, cols, SRU_AMD_F32, SRU_AMD_F32) != SRU_AMD_OK) return 0;
-    return (size_t)norm_blocks(rows) * 2 * (size_t)cols * sizeof(float);
+    // one float row pair per workgroup of the backward kernel, then the slabs of the two-launch sum
+    return (size_t)norm_blocks(rows) * 2 * (size_t)cols * sizeof(float) + (size_t)kSlabs * 2 * (size_t)cols * sizeof(double);
 }
 
 int sru_amd_layer_norm_backward(int64_t rows, int64_t cols, const void *x, int x_dtype, const float *weight,
@@ -333,9 +426,24 @@ int sru_amd_layer_norm_backward(int64_t rows, int64_t cols, const void *x, int x
     if (err != hipSuccess) return SRU_AMD_ERR_LAUNCH;
     int32_t nrows = norm_blocks(rows), width = 2 * D;
     const float *src = partial;
-    void *args[] = {&src, &grad_weight, &nrows, &width};
-    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows), dim3((width + kLanes - 1) / kLanes),
-                           dim3(kLanes * kRowSlices), args, 0, st) == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+    const dim3 columns((width + kLanes - 1) / kLanes), threads(kLanes * kRowSlices);
+    if (nrows <= 4 * kSlabs) {
+        int32_t chunk = nrows;
+        void *args[] = {&src, &grad_weight, &nrows, &width, &chunk};
+        return hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows<float, float>), columns, threads, args, 0, st) ==
+                       hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+    }
+    double *slabs = reinterpret_cast<double *>(partial + (size_t)nrows * width);
+    int32_t chunk = (nrows + kSlabs - 1) / kSlabs;
+    void *first[] = {&src, &slabs, &nrows, &width, &chunk};
+    if (hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows<float, double>), dim3(columns.x, kSlabs), threads, first,
+                        0, st) != hipSuccess)
+        return SRU_AMD_ERR_LAUNCH;
+    const double *mid = slabs;
+    int32_t nslabs = kSlabs, all = kSlabs;
+    void *second[] = {&mid, &grad_weight, &nslabs, &width, &all};
+    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows<double, float>), columns, threads, second, 0, st) ==
+                   hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
 }
 
 }  // extern "C"

@@ -106,8 +106,9 @@ def test_layer_norm_entry_points_validate_before_launching():
     assert fwd(4, 64, x=None) == 1
     assert fwd(4, 64, x=ctypes.c_void_p(0x1004)) == 5
     need = lib.sru_amd_layer_norm_backward_workspace_bytes(4, 64)
-    assert need == 1 * 2 * 64 * 4 and lib.sru_amd_layer_norm_backward_workspace_bytes(4, 12) == 0
-    assert lib.sru_amd_layer_norm_backward_workspace_bytes(10 ** 6, 1024) == 1024 * 2 * 1024 * 4
+    slabs = 16 * 2 * 8    # bytes per feature of the second stage of the sum over workgroups
+    assert need == 2 * 2 * 64 * 4 + slabs * 64 and lib.sru_amd_layer_norm_backward_workspace_bytes(4, 12) == 0
+    assert lib.sru_amd_layer_norm_backward_workspace_bytes(10 ** 6, 1024) == 1024 * 2 * 1024 * 4 + slabs * 1024
     gw = ctypes.c_void_p(0x2000)
     gb = ctypes.c_void_p(0x2000 + 64 * 4)
     bwd = lambda ws, nbytes, gbias=gb: lib.sru_amd_layer_norm_backward(
