@@ -383,8 +383,22 @@ def main():
     # What the selected kernels are built to move: with checkpoints the per-step state (es bytes per
     # cell each way) shrinks to one float per 8 steps.
     state_bytes = (4 * cells // 8) if ckpt else es * cells
-    fwd_moved = (k + (1 if use_x else 0) + 1 + (2 if custom else 0)) * es * cells + (0 if fwd_only else state_bytes)
-    bwd_moved = (2 * k + (2 if use_x else 0) + 1 + (4 if custom else 0)) * es * cells + state_bytes
+    # Padding at the ends of a batch row's sequence is skipped in chunks of 8 steps by the kernels
+    # whose wavefronts lie inside one batch row: those cells cost their output bytes only.
+    live_f = live_b = 1.0
+    if padded:
+        walked = torch.clamp((lens + 7) // 8 * 8, max=L).sum().item() / float(L * B)
+        sixteen = es == 2
+        lane_pairs = (sixteen and d % 32 == 0 and ncols // 32 <= 1024 and os.environ.get("SRU_AMD_SPLIT") != "0"
+                      and (ckpt or fwd_only))          # those kernels walk every step
+        cols = 2 if sixteen and ncols // 2 >= 65536 else 1
+        uniform = d % (64 * cols) == 0 and not lane_pairs and not (custom and args.tanh)
+        live_f = walked if uniform else 1.0
+        live_b = walked if uniform and ckpt else 1.0   # (the state-after-every-step backward kernel walks every step)
+    fwd_in = (k + (1 if use_x else 0) + (2 if custom else 0)) * es * cells
+    bwd_in = (k + (1 if use_x else 0) + 1 + (2 if custom else 0)) * es * cells + state_bytes
+    fwd_moved = int(fwd_in * live_f) + es * cells + (0 if fwd_only else state_bytes)
+    bwd_moved = int(bwd_in * live_b) + (k + (1 if use_x else 0) + (2 if custom else 0)) * es * cells
     if fwd_only:
         bwd_us = float("nan")
     bwd_gbs = bwd_bytes / (bwd_us * 1e-6) / 1e9
@@ -409,6 +423,7 @@ def main():
                      "algorithmic_bytes_per_launch": bwd_bytes,
                      "moved_bytes_per_launch": bwd_moved,
                      "moved_frac": gbs(bwd_moved, bwd_us) / HBM_PEAK_GBS,
+                     "walked_cell_fraction": {"forward": live_f, "backward": live_b},
                      "note": "achieved / frac price the reference algorithm's bytes (state after every step written "
                              "and read); moved_* price what the selected kernels move (state checkpoints), "
                              "actual_frac the counter-measured traffic",

@@ -510,6 +510,32 @@ __global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
     for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
 }
 
+// Window of a wavefront's walk outside of which every step is padded, for wavefronts whose lanes
+// share one batch row (kUniform): [lo, hi) in walk steps, lo = hi = 0 when the whole row is
+// padding. Lane l looks at steps l, l + 64, ...; the flags of any mask are honoured inside the
+// window, so only leading and trailing padding is skipped (right-padded batches: the tail of the
+// forward direction's walk, the head of the reverse direction's).
+struct LiveWindow { int64_t lo, hi; };
+__device__ __forceinline__ LiveWindow live_window(const uint8_t *pad, int64_t pf, int64_t ps, int64_t L) {
+    if (L >= (INT64_C(1) << 30)) return {0, L};
+    int lo = (int)L, hi = 0;
+#pragma unroll 8
+    for (int s = (int)threadIdx.x; s < (int)L; s += kBlock) {
+        const bool live = pad[pf + s * ps] == 0;
+        lo = live ? min(lo, s) : lo;
+        hi = live ? max(hi, s + 1) : hi;
+    }
+#pragma unroll
+    for (int off = kBlock / 2; off > 0; off >>= 1) {
+        lo = min(lo, __shfl_xor(lo, off, kBlock));
+        hi = max(hi, __shfl_xor(hi, off, kBlock));
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    if (hi <= lo) return {0, 0};
+    return {lo, hi};
+}
+
 // ================================================================= forward scan, chunked
 // Same results as forward_scan. Instead of a ring refilled step by step, the walk is cut
 // into chunks of TC steps held in two alternating register sets: the loads of chunk n+1
@@ -639,13 +665,36 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
         }
     };
 
+    // steps the window leaves out are known to be padded: no loads, the outputs a padded step gets
+    auto fill = [&](int64_t from, int64_t to) __attribute__((always_inline)) {
+        const float zero[COLS] = {};
+        for (int64_t s = from; s < to; ++s) {
+            const int64_t e = ef + s * es;
+            S1::template store<NTS>(hbase + e, lane, q, zero);
+            if (KEEP_C) S1::template store<NTS>(cbase + e, lane, q, cur);
+            if (CKPT && s % TC == TC - 1) {
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) p.ckpt[(s / TC) * p.ncols + col + c] = cur[c];
+            }
+        }
+    };
+
     const int64_t nfull = L / TC;
     const int tail = (int)(L - nfull * TC);
+    int64_t ch = 0, nend = nfull;   // full chunks [ch, nend) are walked
+    bool with_tail = tail > 0;      // and the ragged last chunk
+    if constexpr (HAS_PAD && UNI) {
+        const LiveWindow w = live_window(p.pad, pf, ps, L);
+        ch = w.lo / TC;
+        const int64_t chunks = (w.hi + TC - 1) / TC;
+        nend = chunks < nfull ? chunks : nfull;
+        with_tail = with_tail && chunks > nfull;
+        fill(0, ch * TC);
+    }
     Chunk ka, kb;
-    int64_t ch = 0;
-    if (nfull > 0) load_chunk(ka, 0, TC);
+    if (ch < nend) load_chunk(ka, ch, TC);
     // two chunks per iteration: every prefetch inside the loop is a real chunk
-    while (ch + 2 < nfull) {
+    while (ch + 2 < nend) {
         load_chunk(kb, ch + 1, TC);
         __builtin_amdgcn_sched_barrier(0);  // all loads of the next chunk first, then the arithmetic
         compute_chunk(ka, ch, TC);
@@ -657,20 +706,21 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
         ch += 2;
     }
     // one or two full chunks remain (ka holds chunk ch), then the ragged tail
-    if (ch + 1 < nfull) {
+    if (ch + 1 < nend) {
         load_chunk(kb, ch + 1, TC);
         compute_chunk(ka, ch, TC);
-        if (tail > 0) load_chunk(ka, nfull, tail);
+        if (with_tail) load_chunk(ka, nfull, tail);
         compute_chunk(kb, ch + 1, TC);
-        if (tail > 0) compute_chunk(ka, nfull, tail);
-    } else if (ch < nfull) {
-        if (tail > 0) load_chunk(kb, nfull, tail);
+        if (with_tail) compute_chunk(ka, nfull, tail);
+    } else if (ch < nend) {
+        if (with_tail) load_chunk(kb, nfull, tail);
         compute_chunk(ka, ch, TC);
-        if (tail > 0) compute_chunk(kb, nfull, tail);
-    } else if (tail > 0) {
+        if (with_tail) compute_chunk(kb, nfull, tail);
+    } else if (with_tail) {
         load_chunk(kb, nfull, tail);
         compute_chunk(kb, nfull, tail);
     }
+    if constexpr (HAS_PAD && UNI) fill(with_tail ? L : nend * TC, L);
 #pragma unroll
     for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
 }
@@ -1034,18 +1084,39 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         }
     };
 
+    // steps the window leaves out are known to be padded: no loads, zero gradients
+    auto fill = [&](int64_t from, int64_t to) __attribute__((always_inline)) {
+        const float zu[COLS * K] = {}, z1[COLS] = {}, zv[COLS * 2] = {};
+        for (int64_t s = from; s < to; ++s) {
+            const int64_t e = ef + s * es;
+            SU::template store<NTS>(gubase + e * K, lane, q, zu);
+            if (SKIP == 1) S1::template store<NTS>(gxbase + e, lane, q, z1);
+            if constexpr (CUSTOM) SV::template store<NTS>(gvbase + e * 2, lane, q, zv);
+        }
+    };
+
     const int64_t nfull = L / TC;
     const int tail = (int)(L - nfull * TC);
+    int64_t first = 0, nend = nfull;   // full chunks [first, nend) are walked, last to first
+    bool with_tail = tail > 0;         // and, before them, the ragged last chunk
+    if constexpr (HAS_PAD && UNI) {
+        const LiveWindow w = live_window(p.pad, pf, ps, L);
+        first = w.lo / TC;
+        const int64_t chunks = (w.hi + TC - 1) / TC;
+        nend = chunks < nfull ? chunks : nfull;
+        with_tail = with_tail && chunks > nfull;
+        fill(with_tail ? L : nend * TC, L);
+    }
     Chunk ka, kb;
-    int64_t ch = nfull - 1;           // next full chunk to compute
-    if (ch >= 0) load_chunk(ka, ch, TC);
-    if (tail > 0) {                    // the ragged chunk is the last of the walk: visited first
+    int64_t ch = nend - 1;             // next full chunk to compute
+    if (ch >= first) load_chunk(ka, ch, TC);
+    if (with_tail) {                   // the ragged chunk is the last of the walk: visited first
         load_chunk(kb, nfull, tail);
         compute_chunk(kb, nfull, tail);
     }
     // Two chunks per iteration (ka, kb alternate) so that no register copies are needed and
     // the loop body is a single block in which every prefetch is a real chunk.
-    while (ch >= 2) {
+    while (ch >= first + 2) {
         load_chunk(kb, ch - 1, TC);
         compute_chunk(ka, ch, TC);
         __builtin_amdgcn_sched_barrier(0);
@@ -1054,13 +1125,14 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
         __builtin_amdgcn_sched_barrier(0);
         ch -= 2;
     }
-    if (ch == 1) {
-        load_chunk(kb, 0, TC);
-        compute_chunk(ka, 1, TC);
-        compute_chunk(kb, 0, TC);
-    } else if (ch == 0) {
-        compute_chunk(ka, 0, TC);
+    if (ch == first + 1) {
+        load_chunk(kb, first, TC);
+        compute_chunk(ka, first + 1, TC);
+        compute_chunk(kb, first, TC);
+    } else if (ch == first) {
+        compute_chunk(ka, first, TC);
     }
+    if constexpr (HAS_PAD && UNI) fill(0, first * TC);
 
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {

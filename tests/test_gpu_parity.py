@@ -274,3 +274,44 @@ def test_saturated_gates_stay_finite(checkpointed, act):
     hit.reshape(c.L, c.B, c.Dp, c.k)[..., 0] = False      # gate streams only; u0 stays moderate
     c.U = np.where(hit, big, c.U)
     check_against_oracle(c.f32(), "f32", checkpointed=checkpointed)
+
+
+def _windowed_mask(L, B, kind, rng):
+    """Masks whose padding sits at the ends of the sequences, where the wave-uniform kernels skip
+    whole chunks of 8 steps: every batch row gets a live span [lo, hi) of its own."""
+    pad = np.ones((L, B), bool)
+    for b in range(B):
+        if kind == "right":
+            lo, hi = 0, int(rng.integers(1, L + 1))
+        elif kind == "left":
+            lo, hi = int(rng.integers(0, L)), L
+        elif kind == "both":
+            lo = int(rng.integers(0, L - 1))
+            hi = int(rng.integers(lo + 1, L + 1))
+        elif kind == "chunk_edges":            # spans that start and end on multiples of 8
+            lo = 8 * int(rng.integers(0, L // 8))
+            hi = min(L, lo + 8 * int(rng.integers(1, L // 8 + 1)))
+        else:                                  # "holes": live ends, padding inside the span too
+            lo, hi = int(rng.integers(0, L // 2)), int(rng.integers(L // 2 + 1, L + 1))
+        pad[lo:hi, b] = False
+        if kind == "holes":
+            inner = rng.random(hi - lo) < 0.4
+            inner[0] = inner[-1] = False
+            pad[lo:hi, b] |= inner
+    if kind in ("both", "holes"):
+        pad[:, B - 1] = True                   # one batch row with no live step at all
+    return pad
+
+
+@pytest.mark.parametrize("dt,checkpointed", [("f32", False), ("f32", True), ("bf16", True), ("f16", False)])
+@pytest.mark.parametrize("kind", ["right", "left", "both", "chunk_edges", "holes"])
+@pytest.mark.parametrize("L", [64, 45])
+def test_padding_at_the_ends_of_sequences_is_skipped_exactly(L, kind, dt, checkpointed):
+    rng = np.random.default_rng(L + len(kind))
+    for cfg in (dict(B=5, d=128, dirs=2), dict(B=3, d=256, dirs=1, k=4), dict(B=4, d=128, dirs=2, mask_c=True, scale=1.7)):
+        c = Case(L=L, seed=61, **cfg)
+        c.pad = _windowed_mask(L, c.B, kind, rng)
+        check_against_oracle(c, dt, checkpointed=checkpointed)
+    c = Case(L=L, B=4, d=128, dirs=2, seed=62)
+    c.pad = _windowed_mask(L, 4, kind, rng)
+    check_against_oracle(c, dt, keep_c=False)
