@@ -10,6 +10,7 @@
 // clears the runtime's sticky error state, which may hold an error of the embedding program.
 #pragma once
 
+#include <algorithm>
 #include <cstdlib>
 
 #include "sru_launch.h"
@@ -41,15 +42,28 @@ inline bool split_wanted(int64_t ncols, int32_t d) {
 
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-inline dim3 grid_for(int64_t ncols, int cols) {
-    const int64_t lanes = ncols / cols;
-    return dim3((unsigned)((lanes + kBlock - 1) / kBlock));
-}
-
 template <typename P>
 inline hipError_t launch(void (*kernel)(P), dim3 grid, hipStream_t st, const P &p) {
     void *args[] = {const_cast<P *>(&p)};
     return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, dim3(kBlock), args, 0, st);
+}
+
+// Wavefronts per workgroup for the chunked kernels: 8 or 4 (as the kernel allows) while the launch
+// still has a workgroup for each of the 256 compute units, else 1. (Not 2: workgroups of two
+// wavefronts measured up to 25 % slower than either neighbour.)
+inline int waves_per_group(int64_t wavefronts, int most) {
+    for (int n = most; n >= 4; n /= 2)
+        if (wavefronts / n >= 256) return n;
+    return 1;
+}
+// launch of a chunked kernel: `most` wavefronts per workgroup at most
+template <typename P>
+inline hipError_t launch_grouped(void (*kernel)(P), int64_t ncols, int cols, int most, hipStream_t st, const P &p) {
+    const int64_t wavefronts = (ncols / cols + kBlock - 1) / kBlock;
+    const int n = waves_per_group(wavefronts, most);
+    void *args[] = {const_cast<P *>(&p)};
+    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), dim3((unsigned)((wavefronts + n - 1) / n)), dim3(kBlock * n),
+                           args, 0, st);
 }
 
 // Two columns per lane need an even d (a pair must not straddle a direction or a batch
@@ -84,13 +98,13 @@ hipError_t fast_forward(const FwdParams &p, hipStream_t st) {
         return p.pad ? fast_forward<T, K, SKIP, COLS, X | kHasPad, 3>(p, st) : fast_forward<T, K, SKIP, COLS, X, 3>(p, st);
     } else {
         constexpr int TC = kCkptInterval;
-        const dim3 grid = grid_for(p.ncols, COLS);
+        const int most = max_waves_per_group<T>(X);
         // what is kept for the backward pass: checkpoints, the state after every step, or nothing
-        if (p.ckpt) return launch(forward_scan_chunked<T, K, SKIP, X | kNt | kCkpt, COLS, TC>, grid, st, p);
+        if (p.ckpt) return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt | kCkpt, COLS, TC>, p.ncols, COLS, most, st, p);
         if constexpr ((X & kCustom) == 0) {   // (with a per-step weight_c the state after every step is the general kernels')
-            if (p.c) return launch(forward_scan_chunked<T, K, SKIP, X | kNt | kKeepC, COLS, TC>, grid, st, p);
+            if (p.c) return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt | kKeepC, COLS, TC>, p.ncols, COLS, most, st, p);
         }
-        return launch(forward_scan_chunked<T, K, SKIP, X | kNt, COLS, TC>, grid, st, p);
+        return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt, COLS, TC>, p.ncols, COLS, most, st, p);
     }
 }
 
@@ -103,14 +117,15 @@ hipError_t fast_backward(const BwdParams &p, hipStream_t st) {
     } else if constexpr (STAGE == 1) {
         return p.pad ? fast_backward<T, K, SKIP, COLS, X | kHasPad, 2>(p, st) : fast_backward<T, K, SKIP, COLS, X, 2>(p, st);
     } else {
-        const dim3 grid = grid_for(p.ncols, COLS);
         if constexpr ((X & (kPair | kCustom)) == 0) {   // (lane pairing and the weight_c stream exist in the chunked kernels only)
             // reference-style state: the ring kernel reads it step by step
-            if (!p.ckpt) return launch(backward_scan<T, K, SKIP, X | kNt, COLS, kRingDepth>, grid, st, p);
+            if (!p.ckpt) return launch_grouped(backward_scan<T, K, SKIP, X | kNt, COLS, kRingDepth>, p.ncols, COLS, 4, st, p);
         }
         constexpr int TC = kCkptInterval;
-        if (wave_uniform(p.d, COLS)) return launch(backward_scan_ckpt<T, K, SKIP, X | kNt | kUniform, COLS, TC>, grid, st, p);
-        return launch(backward_scan_ckpt<T, K, SKIP, X | kNt, COLS, TC>, grid, st, p);
+        const int most = max_waves_per_group<T>(X);
+        if (wave_uniform(p.d, COLS))
+            return launch_grouped(backward_scan_ckpt<T, K, SKIP, X | kNt | kUniform, COLS, TC>, p.ncols, COLS, most, st, p);
+        return launch_grouped(backward_scan_ckpt<T, K, SKIP, X | kNt, COLS, TC>, p.ncols, COLS, most, st, p);
     }
 }
 
@@ -146,11 +161,11 @@ inline bool all_aligned_16(std::initializer_list<const void *> ptrs) {
 
 template <typename T, int K, int SKIP>
 hipError_t general_forward(const FwdParams &p, hipStream_t st) {
-    return launch(forward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, grid_for(p.ncols, 1), st, p);
+    return launch_grouped(forward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, p.ncols, 1, 4, st, p);
 }
 template <typename T, int K, int SKIP>
 hipError_t general_backward(const BwdParams &p, hipStream_t st) {
-    return launch(backward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, grid_for(p.ncols, 1), st, p);
+    return launch_grouped(backward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, p.ncols, 1, 4, st, p);
 }
 
 // 16-bit streams whose columns cannot be paired (odd d, or a stream pointer that is not aligned to a

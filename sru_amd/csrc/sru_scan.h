@@ -22,7 +22,15 @@
 
 namespace sru_amd {
 
-constexpr int kBlock = 64;  // one wavefront per workgroup: finest dispatch granularity
+constexpr int kBlock = 64;  // lanes of a wavefront; a wavefront is the unit of work of every kernel
+// Wavefronts per workgroup of the chunked kernels (nothing is shared between them). Neighbouring
+// wavefronts own neighbouring columns; in one workgroup they start together on one compute unit and
+// stay close in time, so their 256- and 768-byte row segments reach memory as longer runs.
+// (Four at most, one per SIMD, leave every wavefront the whole register file; the plain float
+// kernels fit eight.)
+template <typename T> constexpr int max_waves_per_group(int mode) {
+    return (sizeof(T) == 4 && (mode & (256 | 512)) == 0) ? 8 : 4;
+}
 
 struct half_bits { uint16_t v; };  // IEEE binary16 storage
 struct bf16_bits { uint16_t v; };  // bfloat16 storage
@@ -386,11 +394,11 @@ struct CompensatedSum {
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
 // U[..., 3]. COLS: columns per lane (2 needs an even d). P: ring depth.
 template <typename T, int K, int SKIP, int MODE, int COLS, int P>
-__global__ void __launch_bounds__(kBlock) forward_scan(const FwdParams p) {
+__global__ void __launch_bounds__(kBlock * 4) forward_scan(const FwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     static_assert((MODE & (kCkpt | kPair | kUniform)) == 0, "those exist in the chunked kernels only");
-    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;  // lane's first column
+    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * COLS;  // lane's first column
     if (col >= p.ncols) return;
 
     const int Dp = p.Dp;
@@ -520,7 +528,7 @@ __device__ __forceinline__ LiveWindow live_window(const uint8_t *pad, int64_t pf
     if (L >= (INT64_C(1) << 30)) return {0, L};
     int lo = (int)L, hi = 0;
 #pragma unroll 8
-    for (int s = (int)threadIdx.x; s < (int)L; s += kBlock) {
+    for (int s = (int)(threadIdx.x % kBlock); s < (int)L; s += kBlock) {
         const bool live = pad[pf + s * ps] == 0;
         lo = live ? min(lo, s) : lo;
         hi = live ? max(hi, s + 1) : hi;
@@ -545,7 +553,7 @@ __device__ __forceinline__ LiveWindow live_window(const uint8_t *pad, int64_t pf
 // every call site: a chunk that is passed by reference to a real function lives in scratch
 // memory instead of registers.)
 template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
-__global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p) {
+__global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward_scan_chunked(const FwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     static_assert(TC == kCkptInterval, "a chunk is one checkpoint interval");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
@@ -562,10 +570,12 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
     using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c: two elements per column
-    const uint32_t wg = blockIdx.x;
-    const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
+    // the wavefront's index in the launch (scalar), and the lane's in the wavefront
+    const uint32_t wg = blockIdx.x * (blockDim.x / kBlock) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kBlock));
+    const uint32_t wlane = threadIdx.x % kBlock;
+    const int64_t col = ((int64_t)wg * kBlock + wlane) * COLS;
     if (col >= p.ncols) return;
-    const int q = PAIR ? (int)(threadIdx.x & 1) : 0;  // columns of a pair are col - q, col - q + 1
+    const int q = PAIR ? (int)(wlane & 1) : 0;  // columns of a pair are col - q, col - q + 1
 
     // colu decides direction and batch row: the wavefront's first column when that is the same
     // for all its lanes (scalar), else the lane's own column
@@ -622,7 +632,7 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
         }
         // one load for the whole chunk: lane l fetches the flag of step l % TC (clamped to the
         // chunk's last valid step), compute_chunk reads step i's flag from lane i
-        if (PAD_BY_LANE) k.pad[0] = p.pad[pf + (s0 + min((int)(threadIdx.x % TC), n - 1)) * ps];
+        if (PAD_BY_LANE) k.pad[0] = p.pad[pf + (s0 + min((int)(wlane % TC), n - 1)) * ps];
     };
 
     auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
@@ -731,10 +741,10 @@ __global__ void __launch_bounds__(kBlock) forward_scan_chunked(const FwdParams p
 // gradients over time stay in registers and leave the kernel as per-column partials;
 // reduce_partials() then adds them over the batch in a fixed order.
 template <typename T, int K, int SKIP, int MODE, int COLS, int P>
-__global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
+__global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
-    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * COLS;
+    const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
 
     const int Dp = p.Dp;
@@ -922,7 +932,7 @@ __global__ void __launch_bounds__(kBlock) backward_scan(const BwdParams p) {
 // arithmetic of the current one. Per cell: reads U (k), x, grad_h and 4/TC bytes of
 // checkpoint; writes grad_u (k), grad_x.
 template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
-__global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) {
+__global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backward_scan_ckpt(const BwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
@@ -932,10 +942,12 @@ __global__ void __launch_bounds__(kBlock) backward_scan_ckpt(const BwdParams p) 
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
     using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c and its gradient: two elements per column
-    const uint32_t wg = blockIdx.x;
-    const int64_t col = ((int64_t)wg * kBlock + threadIdx.x) * COLS;
+    // the wavefront's index in the launch (scalar), and the lane's in the wavefront
+    const uint32_t wg = blockIdx.x * (blockDim.x / kBlock) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kBlock));
+    const uint32_t wlane = threadIdx.x % kBlock;
+    const int64_t col = ((int64_t)wg * kBlock + wlane) * COLS;
     if (col >= p.ncols) return;
-    const int q = PAIR ? (int)(threadIdx.x & 1) : 0;
+    const int q = PAIR ? (int)(wlane & 1) : 0;
 
     const int64_t colu = UNI ? (int64_t)wg * (kBlock * COLS) : col;  // see forward_scan_chunked
     const uint32_t lane = (uint32_t)(col - colu);
