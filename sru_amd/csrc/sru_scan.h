@@ -26,10 +26,10 @@ constexpr int kBlock = 64;  // lanes of a wavefront; a wavefront is the unit of 
 // Wavefronts per workgroup of the chunked kernels (nothing is shared between them). Neighbouring
 // wavefronts own neighbouring columns; in one workgroup they start together on one compute unit and
 // stay close in time, so their 256- and 768-byte row segments reach memory as longer runs.
-// (Four at most, one per SIMD, leave every wavefront the whole register file; the plain float
-// kernels fit eight.)
+// (Four at most, one per SIMD, leave every wavefront the whole register file; the float kernels
+// without a weight_c stream fit eight, i.e. into 256 registers.)
 template <typename T> constexpr int max_waves_per_group(int mode) {
-    return (sizeof(T) == 4 && (mode & (256 | 512)) == 0) ? 8 : 4;
+    return (sizeof(T) == 4 && (mode & 512) == 0) ? 8 : 4;
 }
 
 struct half_bits { uint16_t v; };  // IEEE binary16 storage
