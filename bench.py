@@ -232,6 +232,8 @@ def main():
                          "reference's custom_m returning V)")
     ap.add_argument("--torch-layer-norm", action="store_true",
                     help="with a stack workload: use torch.nn.LayerNorm's kernels instead of this package's")
+    ap.add_argument("--shape", default=None, metavar="L,B,d,dirs",
+                    help="side measurement at another shape (k=3 forward + backward, no padding); replaces --workload")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "
@@ -253,6 +255,9 @@ def main():
         return None if t is None else ctypes.c_void_p(t.data_ptr())
 
     name, L, B, d, dirs, k, fwd_only, padded = WORKLOADS[args.workload]
+    if args.shape:
+        L, B, d, dirs = (int(v) for v in args.shape.split(","))
+        name, k, fwd_only, padded = f"{'bi' if dirs == 2 else 'uni'}-SRU d={d} L={L} B={B} k=3", 3, False, False
     name += " " + args.dtype
     Dp = d * dirs
     ncols, cells = B * Dp, L * B * Dp

@@ -42,10 +42,13 @@ inline bool split_wanted(int64_t ncols, int32_t d) {
 
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// launch of a lane-pair kernel: wavefronts of 32 columns, kSplitWaves per workgroup
 template <typename P>
-inline hipError_t launch(void (*kernel)(P), dim3 grid, hipStream_t st, const P &p) {
+inline hipError_t launch_split(void (*kernel)(P), hipStream_t st, const P &p) {
     void *args[] = {const_cast<P *>(&p)};
-    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, dim3(kBlock), args, 0, st);
+    const int64_t wavefronts = p.ncols / kSplitCols;
+    return hipLaunchKernel(reinterpret_cast<const void *>(kernel), dim3((unsigned)((wavefronts + kSplitWaves - 1) / kSplitWaves)),
+                           dim3(kBlock * kSplitWaves), args, 0, st);
 }
 
 // Wavefronts per workgroup for the chunked kernels: 8 or 4 (as the kernel allows) while the launch
@@ -136,9 +139,8 @@ hipError_t split_forward(const FwdParams &p, hipStream_t st) {
     } else if constexpr (STAGE == 1) {
         return p.pad ? split_forward<T, K, SKIP, X | kHasPad, 2>(p, st) : split_forward<T, K, SKIP, X, 2>(p, st);
     } else {
-        const dim3 grid((unsigned)(p.ncols / kSplitCols));
-        if (p.ckpt) return launch(forward_scan_split<T, K, SKIP, X | kNt | kCkpt, kSplitNbuf>, grid, st, p);
-        return launch(forward_scan_split<T, K, SKIP, X | kNt, kSplitNbuf>, grid, st, p);
+        if (p.ckpt) return launch_split(forward_scan_split<T, K, SKIP, X | kNt | kCkpt, kSplitNbuf>, st, p);
+        return launch_split(forward_scan_split<T, K, SKIP, X | kNt, kSplitNbuf>, st, p);
     }
 }
 
@@ -147,9 +149,8 @@ hipError_t split_backward(const BwdParams &p, hipStream_t st) {
     if constexpr (STAGE == 0) {
         return p.act ? split_backward<T, K, SKIP, X | kTanh, 1>(p, st) : split_backward<T, K, SKIP, X, 1>(p, st);
     } else {
-        const dim3 grid((unsigned)(p.ncols / kSplitCols));
-        if (p.pad) return launch(backward_scan_split<T, K, SKIP, X | kNt | kHasPad, kSplitNbuf>, grid, st, p);
-        return launch(backward_scan_split<T, K, SKIP, X | kNt, kSplitNbuf>, grid, st, p);
+        if (p.pad) return launch_split(backward_scan_split<T, K, SKIP, X | kNt | kHasPad, kSplitNbuf>, st, p);
+        return launch_split(backward_scan_split<T, K, SKIP, X | kNt, kSplitNbuf>, st, p);
     }
 }
 

@@ -23,7 +23,10 @@
 namespace sru_amd {
 
 constexpr int kSplitCols = 32;    // columns per wavefront
-constexpr int kSplitChunk = 16;   // steps per chunk: two checkpoint intervals
+constexpr int kSplitChunk = 16;
+// Wavefronts per workgroup (independent of each other): four land on the four SIMDs of a compute
+// unit, where single-wavefront workgroups leave some SIMDs with two wavefronts and others with none.
+constexpr int kSplitWaves = 4;   // steps per chunk: two checkpoint intervals
 
 // value of the other lane of the pair (quad_perm [1,0,3,2])
 __device__ __forceinline__ float pair_swap(float v) {
@@ -69,7 +72,7 @@ struct SplitTile {
 // allocator is told not to save registers for an occupancy that will not happen: with its default
 // target of four it serialised the LDS reads of a chunk through one register.)
 template <typename T, int K, int SKIP, int MODE, int NBUF>
-__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(1, 2)))
+__global__ void __launch_bounds__(kBlock * kSplitWaves) __attribute__((amdgpu_waves_per_eu(1, 2)))
 forward_scan_split(const FwdParams p) {
     static_assert(sizeof(T) == 2, "16-bit streams");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
@@ -79,13 +82,18 @@ forward_scan_split(const FwdParams p) {
     using T1 = typename G::T1;
     constexpr int TC = G::TC, W = G::W, PITCH = G::kPitch;
     static_assert(TC == 2 * kCkptInterval, "a chunk is two checkpoint intervals");
-    __shared__ __attribute__((aligned(16))) unsigned char lds_in[G::kBytes];
-    __shared__ __attribute__((aligned(16))) unsigned char lds_h[2 * T1::kBytes];   // h tile, then role 0's dump tile
-    __shared__ uint32_t lds_pad[kBlock];
+    __shared__ __attribute__((aligned(16))) unsigned char all_in[kSplitWaves][G::kBytes];
+    __shared__ __attribute__((aligned(16))) unsigned char all_h[kSplitWaves][2 * T1::kBytes];   // h tile, then role 0's dump tile
+    __shared__ uint32_t all_pad[kSplitWaves][kBlock];
+    // the wavefronts of a workgroup share nothing: each has its own tiles and its own 32 columns
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kBlock));
+    unsigned char *lds_in = all_in[wave], *lds_h = all_h[wave];
+    uint32_t *lds_pad = all_pad[wave];
 
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x % kBlock;
     const int c = lane >> 1, role = lane & 1;
-    const int64_t colu = (int64_t)blockIdx.x * W;   // the wavefront's first column (ncols is a multiple of 32)
+    const int64_t colu = ((int64_t)blockIdx.x * kSplitWaves + wave) * W;   // the wavefront's first column (ncols is a multiple of 32)
+    if (colu >= p.ncols) return;
     const int64_t col = colu + c;
     const int Dp = p.Dp;
     const int ju = (int)(colu % Dp);
@@ -218,7 +226,7 @@ forward_scan_split(const FwdParams p) {
 // lane keeps its own gate, the states and its operand A), then the backward recurrence runs over
 // the same steps. The gradient tiles replace the input tile in LDS in place on their way out.
 template <typename T, int K, int SKIP, int MODE, int NBUF>
-__global__ void __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(1, 2)))
+__global__ void __launch_bounds__(kBlock * kSplitWaves) __attribute__((amdgpu_waves_per_eu(1, 2)))
 backward_scan_split(const BwdParams p) {
     static_assert(sizeof(T) == 2, "16-bit streams");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
@@ -228,14 +236,19 @@ backward_scan_split(const BwdParams p) {
     using T1 = typename G::T1;
     constexpr int TC = G::TC, W = G::W, PITCH = G::kPitch;
     // (without a skip term role 1 has no A output: a second tile takes those writes)
-    __shared__ __attribute__((aligned(16))) unsigned char lds_in[G::kBytes * (SKIP == 0 ? 2 : 1)];
-    __shared__ __attribute__((aligned(16))) unsigned char lds_gh[T1::kBytes];
-    __shared__ uint32_t lds_pad[kBlock];
-    __shared__ float lds_cstart[kBlock];
+    __shared__ __attribute__((aligned(16))) unsigned char all_in[kSplitWaves][G::kBytes * (SKIP == 0 ? 2 : 1)];
+    __shared__ __attribute__((aligned(16))) unsigned char all_gh[kSplitWaves][T1::kBytes];
+    __shared__ uint32_t all_pad[kSplitWaves][kBlock];
+    __shared__ float all_cstart[kSplitWaves][kBlock];
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / kBlock));
+    unsigned char *lds_in = all_in[wave], *lds_gh = all_gh[wave];
+    uint32_t *lds_pad = all_pad[wave];
+    float *lds_cstart = all_cstart[wave];
 
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x % kBlock;
     const int c = lane >> 1, role = lane & 1;
-    const int64_t colu = (int64_t)blockIdx.x * W;
+    const int64_t colu = ((int64_t)blockIdx.x * kSplitWaves + wave) * W;
+    if (colu >= p.ncols) return;
     const int64_t col = colu + c;
     const int Dp = p.Dp;
     const int ju = (int)(colu % Dp);
