@@ -11,9 +11,9 @@
 // and the wavefront moves a tile with tile_bytes / 1024 instructions of 1 KB each, whatever a
 // column's share of a row is. A tile passes through LDS to change hands: it is written there in
 // memory order (ds_write_b128) and read back column-wise by the lane that owns the column; outputs
-// go the other way. One wavefront per workgroup owns its LDS tiles alone, and LDS executes a
-// wavefront's instructions in order, so no barrier is needed. The loads of the next chunks are in
-// flight in registers (staging sets, each refilled right after it is drained to LDS).
+// go the other way. A wavefront owns its LDS tiles alone (wavefronts of a workgroup share none), and
+// LDS executes a wavefront's instructions in order, so no barrier is needed. The loads of the next
+// chunks are in flight in registers (staging sets, each refilled right after it is drained to LDS).
 #pragma once
 
 #include "sru_scan.h"
