@@ -208,6 +208,78 @@ def run_stack(args):
                    "layer_norm": "torch" if args.torch_layer_norm else "sru_amd kernels"}}), flush=True)
 
 
+def run_layer_norm(args):
+    """Side measurement: the layer-norm kernels next to the recurrence, through the C ABI, at the
+    row count and width of the headline layer (16 384 rows of 2 048 features). Forward and backward
+    (the backward call includes the two launches that add the workgroups' weight / bias sums) are
+    timed with HIP events on rotating buffer sets; the roofline is HBM, bytes = rows read + written."""
+    import torch
+    from sru_amd import _lib
+    rows, D = 256 * 64, 2048
+    dev = torch.device("cuda:0")
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[args.dtype]
+    code = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}[args.dtype]
+    es = DT_BYTES[args.dtype]
+    lib = _lib.load()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    g = torch.Generator(device=dev).manual_seed(0)
+    w = torch.rand(D, device=dev, generator=g) + 0.5
+    b = torch.randn(D, device=dev, generator=g)
+    nbytes = lib.sru_amd_layer_norm_backward_workspace_bytes(rows, D)
+    sets = []
+    for _ in range(args.sets):
+        sets.append(dict(x=torch.randn(rows, D, device=dev, generator=g).to(tdt), y=torch.empty(rows, D, device=dev, dtype=tdt),
+                         dy=torch.randn(rows, D, device=dev, generator=g).to(tdt), dx=torch.empty(rows, D, device=dev, dtype=tdt),
+                         mean=torch.empty(rows, device=dev), rstd=torch.empty(rows, device=dev),
+                         gwb=torch.empty(2, D, device=dev), ws=torch.empty(nbytes // 4, device=dev)))
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def fwd(s):
+        _lib.check(lib.sru_amd_layer_norm_forward(rows, D, p(s["x"]), code, p(w), p(b), ctypes.c_float(1e-5), p(s["y"]), code,
+                                                  p(s["mean"]), p(s["rstd"]), stream), "sru_amd_layer_norm_forward")
+
+    def bwd(s):
+        _lib.check(lib.sru_amd_layer_norm_backward(rows, D, p(s["x"]), code, p(w), p(s["mean"]), p(s["rstd"]), p(s["dy"]), code,
+                                                   p(s["dx"]), p(s["gwb"][0]), p(s["gwb"][1]), p(s["ws"]),
+                                                   ctypes.c_size_t(nbytes), stream), "sru_amd_layer_norm_backward")
+
+    for s in sets:
+        fwd(s)
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    n = args.warmup + args.steps
+    marks = [(ev(), ev(), ev()) for _ in range(n)]
+    torch.cuda.synchronize()
+    t0 = None
+    for i in range(n):
+        if i == args.warmup:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        a, m, e = marks[i]
+        a.record()
+        fwd(sets[i % args.sets])
+        m.record()
+        bwd(sets[(i + 2) % args.sets])   # a set whose forward ran earlier: operands cache-cold
+        e.record()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    f_us = sum(a.elapsed_time(m) for a, m, _ in marks[args.warmup:]) * 1e3 / args.steps
+    b_us = sum(m.elapsed_time(e) for _, m, e in marks[args.warmup:]) * 1e3 / args.steps
+    f_bytes, b_bytes = 2 * es * rows * D, 3 * es * rows * D
+    gbs = lambda nb, us: nb / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "layer norm rows/s (side measurement)", "value": rows / (ms_step * 1e-3), "unit": "rows/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"workload": f"layer norm forward + backward, {rows} rows of {D} features, {args.dtype} in and out"},
+        "roofline": {"bound": "hbm", "kernel": "layer_norm_backward (+ reduce_rows x 2)", "achieved": gbs(b_bytes, b_us),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs(b_bytes, b_us) / HBM_PEAK_GBS, "traffic": None,
+                     "avg_us": b_us},
+        "kernels": {"layer_norm_forward": {"avg_us": f_us, "algorithmic_GBps": gbs(f_bytes, f_us),
+                                           "frac_of_hbm_peak": gbs(f_bytes, f_us) / HBM_PEAK_GBS},
+                    "layer_norm_backward+reduce": {"avg_us": b_us, "algorithmic_GBps": gbs(b_bytes, b_us),
+                                                   "frac_of_hbm_peak": gbs(b_bytes, b_us) / HBM_PEAK_GBS}}}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,7 +287,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--dtype", default="f32", choices=sorted(DT_BYTES))
     ap.add_argument("--sets", type=int, default=4, help="rotating buffer sets")
-    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + sorted(STACKS))
+    ap.add_argument("--workload", default="headline", choices=sorted(WORKLOADS) + sorted(STACKS) + ["layernorm"])
     ap.add_argument("--full-state", action="store_true",
                     help="keep the state after every step between forward and backward, as the "
                          "reference does, instead of float checkpoints every 8 steps (the path "
@@ -244,6 +316,8 @@ def main():
                  "(columns are independent; no multi-GPU path exists): run with --gpus 1")
     if args.workload in STACKS:
         return run_stack(args)
+    if args.workload == "layernorm":
+        return run_layer_norm(args)
 
     import torch
     from sru_amd import _lib
