@@ -298,7 +298,8 @@ def main():
     ap.add_argument("--tanh", action="store_true",
                     help="side measurement: activation_type = tanh (the reference's deprecated use_tanh)")
     ap.add_argument("--graph", action="store_true",
-                    help="with --workload stack1: record the forward into a HIP graph and time replays")
+                    help="side measurement: record the calls into a HIP graph and time replays (recurrence "
+                         "workloads: one rotation of forward + backward calls; stack1: the forward-only stack)")
     ap.add_argument("--per-step-weight-c", action="store_true",
                     help="side measurement: weight_c given per step, (L, B, D', 2) in the stream dtype (the "
                          "reference's custom_m returning V)")
@@ -384,11 +385,12 @@ def main():
     ws_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(shape))
     ws = torch.empty(ws_bytes // 4, device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    on = [stream]   # the stream the calls are issued on (the capture stream while a graph is recorded)
 
     def fwd(s):
         rc = lib.sru_amd_forward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if use_x else None, p(wc), p(bias),
                                  p(c0), None, p(pad), p(scale) if use_x else None, p(s["h"]),
-                                 None if fwd_only else p(s["c"]), p(c_last), stream)
+                                 None if fwd_only else p(s["c"]), p(c_last), on[0])
         assert rc == 0, _lib.status_string(rc)
 
     def bwd(s):
@@ -397,7 +399,7 @@ def main():
         rc = lib.sru_amd_backward(ctypes.byref(shape), p(s["U"]), p(s["x"]) if use_x else None, p(wc), p(bias),
                                   p(c0), None, p(pad), p(scale) if use_x else None, p(s["c"]), p(s["gh"]),
                                   p(gl), p(s["gu"]), p(s["gx"]) if use_x else None,
-                                  p(gwc), p(gb), p(gi), p(ws), ctypes.c_size_t(ws_bytes), stream)
+                                  p(gwc), p(gb), p(gi), p(ws), ctypes.c_size_t(ws_bytes), on[0])
         assert rc == 0, _lib.status_string(rc)
 
     copy_cal = None
@@ -425,6 +427,35 @@ def main():
     for i in range(args.warmup):
         fwd(sets[i % args.sets])
         bwd(sets[(i + lag) % args.sets])
+    if args.graph:
+        # Side measurement: one rotation of the buffer sets (forward + backward calls) recorded into
+        # a HIP graph and replayed. The entry points neither allocate nor synchronise, so the calls
+        # record as they are; what the replay removes is the host-side gap between dependent launches.
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            on[0] = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+            for i in range(args.sets):
+                fwd(sets[i])
+                bwd(sets[(i + lag) % args.sets])
+        on[0] = stream
+        replays = max(1, args.steps // args.sets)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms_step = (time.perf_counter() - t0) * 1e3 / (replays * args.sets)
+        print(json.dumps({"metric": "recurrence tokens/s, calls replayed from a HIP graph (side measurement)",
+                          "value": L * B / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": replays * args.sets,
+                          "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak",
+                          "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+                          "config": {"workload": name, "pass": "forward only" if fwd_only else "forward+backward, one layer",
+                                     "replayed_from_graph": True, "calls_per_graph": args.sets}}), flush=True)
+        return
     # events live on the stream the kernels are launched on (torch's current stream)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
     torch.cuda.synchronize()
