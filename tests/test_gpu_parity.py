@@ -315,3 +315,17 @@ def test_padding_at_the_ends_of_sequences_is_skipped_exactly(L, kind, dt, checkp
     c = Case(L=L, B=4, d=128, dirs=2, seed=62)
     c.pad = _windowed_mask(L, 4, kind, rng)
     check_against_oracle(c, dt, keep_c=False)
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_long_right_padded_rows_forward_only_and_training(dt):
+    """Many chunks per row, lengths spread over a wide range (the shape class of the L=4096
+    inference configuration, shortened): most wavefronts skip a long tail or head of padding."""
+    rng = np.random.default_rng(77)
+    c = Case(L=523, B=6, d=128, dirs=2, seed=63, scale=1.7)
+    lens = rng.integers(131, 524, c.B)
+    lens[0], lens[1] = 523, 1
+    c.pad = np.arange(c.L)[:, None] >= lens[None, :]
+    check_against_oracle(c, dt, keep_c=False)
+    check_against_oracle(c, dt, checkpointed=True)
+
