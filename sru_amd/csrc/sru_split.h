@@ -261,6 +261,7 @@ backward_scan_split(const BwdParams p) {
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
     // scale of operand A: role 1's skip operand is x * scale_x, U[..., 3], or nothing (times zero)
     const float sa = role ? (SKIP == 0 ? 0.0f : sx) : 1.0f;
+    const float oa_a = role ? m * sx : 1.0f, oa_b = role ? sx : 1.0f;   // see out_a below (sx is 1 unless the skip term is x)
     float cur = p.glast[col];   // d loss / d state (meaningful in role 0)
     CompensatedSum sw, sb;      // the lane's gate: sums of its weight_c and bias gradients
 
@@ -339,11 +340,10 @@ backward_scan_split(const BwdParams p) {
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const bool padded = HAS_PAD && __builtin_amdgcn_readlane((int)padreg, i) != 0;
-                av[i] *= sa;
                 const float b = bv[i];
                 const float cp = st[i];
                 gt[i] = sigmoid_exp2<T>(__builtin_fmaf(knw, cp, __builtin_fmaf(kNegLog2e, b, knb)));
-                const float cn = pair_even((cp - av[i]) * gt[i] + av[i]);
+                const float cn = pair_even((cp - av[i]) * gt[i] + av[i]);   // (role 0's operand A is u0 as it is)
                 st[i + 1] = padded ? cp : cn;
                 vv[i] = role ? (TANH ? tanh_fast(cn) : cn) : cp;
             }
@@ -363,12 +363,14 @@ backward_scan_split(const BwdParams p) {
                 const float to_state = pair_swap(TANH ? ghm * (gg_ * dact) : ghm * gg_);
                 const float gc = to_state + cur;                   // role 0: d loss / d (state after the step)
                 // the lane's gate gradient: role 0 gc * (c_prev - u0) * g1', role 1 gh * m * (val - skip) * g2'
-                const float gate_grad = (role ? ghm : gc) * (vv[i] - av[i]) * d;
+                // (operand A scaled here: role 0 c_prev - u0, role 1 val - x * scale_x)
+                const float gate_grad = (role ? ghm : gc) * __builtin_fmaf(-sa, av[i], vv[i]) * d;
                 const float through_w = gate_grad * w;             // its way back into the previous state
                 const float ncur = gc * gg_ + (through_w + pair_swap(through_w));
-                // outputs A: role 0 grad of the candidate stream; role 1 grad of the skip operand
-                const float skip_grad = gh * (1.0f - gg_ * m);
-                const float out_a = role ? (SKIP == 1 ? skip_grad * sx : skip_grad) : gc * omg;
+                // outputs A: role 0 grad of the candidate stream, gc * (1 - g1); role 1 grad of the skip
+                // operand, gh * (1 - g2 * m) * scale_x: one product of a selected factor and
+                // oa_b - gate * oa_a with per-lane constants
+                const float out_a = (role ? gh : gc) * __builtin_fmaf(-gg_, oa_a, oa_b);
                 lds_put<T>(wa + i * PITCH, padded ? 0.0f : out_a);
                 lds_put<T>(wb + i * PITCH, padded ? 0.0f : gate_grad);
                 gbs += padded ? 0.0f : gate_grad;
