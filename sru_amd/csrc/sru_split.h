@@ -163,11 +163,13 @@ forward_scan_split(const FwdParams p) {
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
                 const bool padded = HAS_PAD && __builtin_amdgcn_readlane((int)padreg, i) != 0;
-                const float a = av[i] * sa, b = bv[i];
+                const float a = av[i], b = bv[i];   // role 0: u0 as it is; role 1: the skip operand before scaling
                 const float g = sigmoid_exp2<T>(__builtin_fmaf(knw, cur, __builtin_fmaf(kNegLog2e, b, knb)));
                 const float cn = pair_even((cur - a) * g + a);      // role 0's result: the new state, to both lanes
                 const float val = TANH ? tanh_fast(cn) : cn;
-                const float out = (SKIP != 0) ? (val - a) * m * g + a : val * m * g;   // role 1's result: h
+                // role 1's result: h = (val - skip) * m * g + skip = val - (val - skip) * (1 - m * g), skip = sa * a
+                const float out = (SKIP != 0) ? __builtin_fmaf(-__builtin_fmaf(-sa, a, val), __builtin_fmaf(-m, g, 1.0f), val)
+                                              : val * m * g;
                 cur = padded ? cur : cn;
                 lds_put<T>(wh + i * T1::kRowBytes, padded ? 0.0f : out);
                 if (CKPT && (i + 1) % kCkptInterval == 0)   // (both lanes of a pair store the same value)
