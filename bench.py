@@ -499,8 +499,7 @@ def main():
     if padded:
         walked = torch.clamp((lens + 7) // 8 * 8, max=L).sum().item() / float(L * B)
         sixteen = es == 2
-        lane_pairs = (sixteen and d % 32 == 0 and ncols // 32 <= 1024 and os.environ.get("SRU_AMD_SPLIT") != "0"
-                      and (ckpt or fwd_only))          # those kernels walk every step
+        lane_pairs = sixteen and d % 32 == 0 and ncols // 32 <= 1024 and (ckpt or fwd_only)   # those kernels walk every step
         cols = 2 if sixteen and ncols // 2 >= 65536 else 1
         uniform = d % (64 * cols) == 0 and not lane_pairs and not (custom and args.tanh)
         live_f = walked if uniform else 1.0

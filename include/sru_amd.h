@@ -32,6 +32,15 @@
  * `dtype` is the element type of the large streams U, x, h, c, grad_h, grad_u,
  * grad_x and of a per-step weight_c / its gradient. The recurrence state and all
  * arithmetic are float whatever `dtype` is.
+ *
+ * Alignment (SRU_AMD_ERR_MISALIGNED otherwise)
+ *   - float tensors: 4 bytes; U and grad_u with k = 4: four elements (one group);
+ *   - every stream: its element size; a per-step weight_c and its gradient: two elements;
+ *   - 16-bit streams with state_interval == SRU_AMD_STATE_INTERVAL move two columns at a
+ *     time: x, h, grad_h, grad_x 4 bytes; U and grad_u 4 bytes (k = 3) or 16 bytes (k = 4);
+ *     a per-step weight_c and its gradient 8 bytes.
+ *   Memory from hipMalloc or a torch allocation satisfies all of these; a view that starts at
+ *   an odd element may not.
  */
 #ifndef SRU_AMD_H
 #define SRU_AMD_H
@@ -43,7 +52,7 @@
 extern "C" {
 #endif
 
-#define SRU_AMD_ABI_VERSION 4
+#define SRU_AMD_ABI_VERSION 5
 
 enum sru_amd_dtype {
     SRU_AMD_F32 = 0,
@@ -55,9 +64,11 @@ enum sru_amd_status {
     SRU_AMD_OK = 0,
     SRU_AMD_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
     SRU_AMD_ERR_BAD_SHAPE = 2,      /* a size is <= 0 or the problem exceeds the index range */
-    SRU_AMD_ERR_BAD_FLAGS = 3,      /* dirs, k, activation_type, skip_type, is_custom inconsistent */
+    SRU_AMD_ERR_BAD_FLAGS = 3,      /* dirs, k, activation_type, skip_type, is_custom inconsistent, or a
+                                     * combination that checkpointed state does not exist for (see
+                                     * state_interval below) */
     SRU_AMD_ERR_BAD_DTYPE = 4,
-    SRU_AMD_ERR_MISALIGNED = 5,     /* a stream pointer is not aligned to its element type */
+    SRU_AMD_ERR_MISALIGNED = 5,     /* a pointer is not aligned as "Alignment" below asks */
     SRU_AMD_ERR_WORKSPACE = 6,      /* workspace missing or smaller than required */
     SRU_AMD_ERR_LAUNCH = 7,         /* the HIP runtime refused the launch */
     SRU_AMD_ERR_STATIC_LIMIT = 8    /* sru_amd_backward_static: more columns than its built-in scratch holds */
@@ -83,8 +94,12 @@ typedef struct sru_amd_shape {
                               * SRU_AMD_STATE_INTERVAL: float checkpoints only, one row per
                               *   SRU_AMD_STATE_INTERVAL steps of each column's walk,
                               *   (max(1, L / SRU_AMD_STATE_INTERVAL), B, D') float; the backward
-                              *   call rebuilds the states in between. Needs is_custom 0 and,
-                              *   with k = 4, a skip term. No counterpart in the reference. */
+                              *   call rebuilds the states in between. Refused (BAD_FLAGS) for
+                              *   k = 4 without a skip term, for is_custom together with tanh, and
+                              *   for 16-bit streams with an odd `hidden`. This is the mode the fast
+                              *   kernels of every shape are built for; with 0 / 1 the 16-bit
+                              *   kernels for few columns and the checkpoint backward kernels are
+                              *   not available. No counterpart in the reference. */
 } sru_amd_shape;
 
 #define SRU_AMD_STATE_INTERVAL 8
@@ -94,6 +109,8 @@ typedef struct sru_amd_shape {
  * :333-412) together with the x * scale_x pass and the gather of the last state
  * that sru/cuda_functional.py:73-78 and :146-153 run around them.
  *   x        required iff skip_type == 1
+ *   c_init   NULL = zeros (what the reference allocates when the caller gives no c0,
+ *            sru/modules.py:241-243)
  *   mask_c   NULL = no dropout mask
  *   mask_pad NULL = no padding
  *   c        state kept for the backward pass, sru_amd_state_bytes() bytes laid out as
@@ -121,6 +138,9 @@ size_t sru_amd_backward_workspace_bytes(const sru_amd_shape *shape);
  * around them: the x * scale_x pass, grad_x *= scale_x and the batch sums of
  * the weight_c / bias gradients.
  *   c         the state buffer the forward call filled (same shape->state_interval)
+ *   c_init    as given to the forward call (NULL = zeros)
+ *   grad_last gradient of c_last; NULL = zeros (the usual case: the last state is not part of
+ *             the loss)
  *   grad_x    required iff skip_type == 1; already multiplied by scale_x
  *   grad_wc   (2, D') float summed over time and batch, or, when is_custom,
  *             (L, B, D', 2) in `dtype`

@@ -3,6 +3,7 @@ with the host-side interface of the reference's sru/cuda_functional.py and sru/o
 from .functional import ElementwiseRecurrence, elementwise_recurrence_forward
 from .ops import elementwise_recurrence_gpu, elementwise_recurrence_inference
 from .modules import SRU, SRUCell
+from .graphs import graphed
 
 __all__ = ["ElementwiseRecurrence", "elementwise_recurrence_forward",
-           "elementwise_recurrence_gpu", "elementwise_recurrence_inference", "SRU", "SRUCell"]
+           "elementwise_recurrence_gpu", "elementwise_recurrence_inference", "SRU", "SRUCell", "graphed"]

@@ -8,9 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# SRU_AMD_LIBRARY points at another build of the same library (tuning builds)
-LIB_PATH = os.environ.get("SRU_AMD_LIBRARY") or os.path.join(_HERE, "libsru_amd.so")
-ABI_VERSION = 4
+LIB_PATH = os.path.join(_HERE, "libsru_amd.so")
+ABI_VERSION = 5
 STATE_INTERVAL = 8   # SRU_AMD_STATE_INTERVAL
 STATIC_MAX_COLUMNS = 262144   # SRU_AMD_STATIC_MAX_COLUMNS
 NORM_MAX_FEATURES = 4096       # SRU_AMD_NORM_MAX_FEATURES

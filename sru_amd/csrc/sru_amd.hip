@@ -88,8 +88,7 @@ int backward_core(const sru_amd_shape *shape, const void *u, const void *x, cons
                   void *grad_u, void *grad_x, void *grad_wc, float *grad_bias, float *grad_init,
                   float *partial, void *stream) {
     const sru_amd_shape &s = *shape;
-    if (!u || !weight_c || !bias || !c_init || !c || !grad_h || !grad_last || !grad_u || !grad_wc ||
-        !grad_bias || !grad_init)
+    if (!u || !weight_c || !bias || !c || !grad_h || !grad_u || !grad_wc || !grad_bias || !grad_init)
         return SRU_AMD_ERR_NULL_POINTER;
     if (s.skip_type == 1 && (!x || !grad_x)) return SRU_AMD_ERR_NULL_POINTER;
     const size_t es = elem_size(s.dtype);
@@ -98,7 +97,7 @@ int backward_core(const sru_amd_shape *shape, const void *u, const void *x, cons
     if (!aligned(u, group) || !aligned(grad_u, group) || !aligned(c, ckpt ? 4 : es) || !aligned(grad_h, es) ||
         (s.skip_type == 1 && (!aligned(x, es) || !aligned(grad_x, es))) ||
         !aligned(weight_c, s.is_custom ? 2 * es : 4) || !aligned(grad_wc, s.is_custom ? 2 * es : 4) ||
-        !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(grad_last, 4) || !aligned(grad_bias, 4) ||
+        !aligned(bias, 4) || (c_init && !aligned(c_init, 4)) || (grad_last && !aligned(grad_last, 4)) || !aligned(grad_bias, 4) ||
         !aligned(grad_init, 4) || (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
         return SRU_AMD_ERR_MISALIGNED;
 
@@ -138,9 +137,10 @@ const char *sru_amd_status_string(int status) {
     case SRU_AMD_OK: return "ok";
     case SRU_AMD_ERR_NULL_POINTER: return "a required pointer is NULL";
     case SRU_AMD_ERR_BAD_SHAPE: return "length, batch or hidden is not positive, or the problem is too large";
-    case SRU_AMD_ERR_BAD_FLAGS: return "inconsistent dirs / k / activation_type / skip_type / is_custom";
+    case SRU_AMD_ERR_BAD_FLAGS:
+        return "inconsistent dirs / k / activation_type / skip_type / is_custom, or checkpointed state asked for a combination it does not exist for";
     case SRU_AMD_ERR_BAD_DTYPE: return "unknown dtype";
-    case SRU_AMD_ERR_MISALIGNED: return "a stream pointer is not aligned to its element group";
+    case SRU_AMD_ERR_MISALIGNED: return "a pointer is not aligned as the header's alignment rules ask";
     case SRU_AMD_ERR_WORKSPACE: return "workspace is NULL, misaligned or too small";
     case SRU_AMD_ERR_LAUNCH: return "the HIP runtime refused the kernel launch";
     case SRU_AMD_ERR_STATIC_LIMIT:
@@ -155,14 +155,14 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
                     void *stream) {
     if (const int rc = check_shape(shape)) return rc;
     const sru_amd_shape &s = *shape;
-    if (!u || !weight_c || !bias || !c_init || !h || !c_last) return SRU_AMD_ERR_NULL_POINTER;
+    if (!u || !weight_c || !bias || !h || !c_last) return SRU_AMD_ERR_NULL_POINTER;
     if (s.skip_type == 1 && !x) return SRU_AMD_ERR_NULL_POINTER;
     const size_t es = elem_size(s.dtype);
     const size_t group = (s.k == 4) ? 4 * es : es;  // a k=4 group moves as one vector
     const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
     if (!aligned(u, group) || !aligned(h, es) || (c && !aligned(c, ckpt ? 4 : es)) ||
         (s.skip_type == 1 && !aligned(x, es)) || !aligned(weight_c, s.is_custom ? 2 * es : 4) ||
-        !aligned(bias, 4) || !aligned(c_init, 4) || !aligned(c_last, 4) ||
+        !aligned(bias, 4) || (c_init && !aligned(c_init, 4)) || !aligned(c_last, 4) ||
         (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
         return SRU_AMD_ERR_MISALIGNED;
 

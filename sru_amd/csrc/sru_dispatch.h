@@ -11,7 +11,6 @@
 #pragma once
 
 #include <algorithm>
-#include <cstdlib>
 
 #include "sru_launch.h"
 #include "sru_split.h"
@@ -29,16 +28,15 @@ constexpr int kRingDepth = 8;  // ring kernels (reference-style state, general m
 constexpr int kNt = kNtLoad | kNtStore;
 // 16-bit streams with few columns: below this many lanes at two columns per lane (fewer than
 // 1024 wavefronts) the kernels keep one column per lane and pair lanes for memory access.
-constexpr int64_t kPairBelow = 65536;
+#ifndef SRU_AMD_PAIR_BELOW   // (set by tuning builds only)
+#define SRU_AMD_PAIR_BELOW 65536
+#endif
+constexpr int64_t kPairBelow = SRU_AMD_PAIR_BELOW;
 
 // Lane-pair kernels (sru_split.h): 16-bit streams, d a multiple of 32, at most 1024 wavefronts of 32
 // columns, every stream 16-byte aligned, state kept as checkpoints or not at all.
 constexpr int kSplitNbuf = 2;   // chunks (of 16 steps) in flight per wavefront
-// SRU_AMD_SPLIT=0 in the environment keeps them out (the one measurement knob; read once)
-inline bool split_wanted(int64_t ncols, int32_t d) {
-    static const bool enabled = [] { const char *e = std::getenv("SRU_AMD_SPLIT"); return !e || std::atoi(e) != 0; }();
-    return enabled && d % kSplitCols == 0 && ncols / kSplitCols <= 1024;
-}
+inline bool split_wanted(int64_t ncols, int32_t d) { return d % kSplitCols == 0 && ncols / kSplitCols <= 1024; }
 
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

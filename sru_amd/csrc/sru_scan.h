@@ -9,9 +9,13 @@
 // pair columns).
 //
 // Latency hiding. The time loop is strictly serial per column (both gates see the
-// previous state), so memory latency is hidden by depth, not by width: every lane keeps
-// a ring of P future steps in registers; each iteration consumes the oldest slot and
-// refills it with the step P ahead.
+// previous state), so memory latency is hidden by depth, not by width. The fast kernels
+// (forward_scan_chunked, backward_scan_ckpt) cut the walk into chunks of 8 steps held in two
+// alternating register sets: the loads of the next chunk are issued in one burst before the
+// arithmetic of the current one. The general kernels and the backward kernel that reads the
+// state after every step (forward_scan, backward_scan) keep a ring of P future steps in
+// registers instead: each iteration consumes the oldest slot and refills it with the step P
+// ahead.
 //
 // Directions. Columns of the second direction walk time backwards. The loop variable
 // is the walk step s (uniform over the wavefront); the time index is s or L-1-s per lane.
@@ -418,7 +422,7 @@ __global__ void __launch_bounds__(kBlock * 4) forward_scan(const FwdParams p) {
         b1[c] = p.bias[j + c];
         b2[c] = p.bias[Dp + j + c];
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
-        cur[c] = p.c0[col + c];
+        cur[c] = p.c0 ? p.c0[col + c] : 0.0f;   // no initial state given: zeros
     }
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
 
@@ -594,7 +598,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
         b1[c] = p.bias[j + c];
         b2[c] = p.bias[Dp + j + c];
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
-        cur[c] = p.c0[col + c];
+        cur[c] = p.c0 ? p.c0[col + c] : 0.0f;   // no initial state given: zeros
     }
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
 
@@ -776,8 +780,8 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
         b1[c] = p.bias[j + c];
         b2[c] = p.bias[Dp + j + c];
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
-        c_init[c] = p.c0[col + c];
-        cur[c] = p.glast[col + c];
+        c_init[c] = p.c0 ? p.c0[col + c] : 0.0f;          // no initial state given: zeros
+        cur[c] = p.glast ? p.glast[col + c] : 0.0f;      // no gradient of the last state given: zeros
         gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
     }
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
@@ -956,7 +960,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
     const int j = ju + (int)lane;
     const bool flip = ju >= p.d;
 
-    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
+    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS];
     float cur[COLS];  // d loss / d state
     CompensatedSum sw1[COLS], sw2[COLS], sb1[COLS], sb2[COLS];  // weight_c / bias gradient sums over the walk
 #pragma unroll
@@ -966,8 +970,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
         b1[c] = p.bias[j + c];
         b2[c] = p.bias[Dp + j + c];
         m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
-        c_init[c] = p.c0[col + c];
-        cur[c] = p.glast[col + c];
+        cur[c] = p.glast ? p.glast[col + c] : 0.0f;      // no gradient of the last state given: zeros
     }
     const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
 
@@ -1010,9 +1013,17 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
         }
+        // one load from a selected address (a select between a register and a loaded value made the
+        // compiler keep the initial state in scratch memory and select between addresses itself)
+        // (without an initial state the first chunk starts from zero; its load reads checkpoint row 0,
+        // which always exists, and drops the value)
+        const bool zero_start = ch == 0 && !p.c0;
+        const float *from = (ch == 0 && p.c0) ? p.c0 + col : p.ckpt + (ch > 0 ? ch - 1 : 0) * p.ncols + col;
 #pragma unroll
-        for (int c = 0; c < COLS; ++c)
-            k.cstart[c] = (ch == 0) ? c_init[c] : p.ckpt[(ch - 1) * p.ncols + col + c];
+        for (int c = 0; c < COLS; ++c) {
+            const float v = from[c];
+            k.cstart[c] = zero_start ? 0.0f : v;
+        }
     };
 
     auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {

@@ -23,10 +23,10 @@
 namespace sru_amd {
 
 constexpr int kSplitCols = 32;    // columns per wavefront
-constexpr int kSplitChunk = 16;
+constexpr int kSplitChunk = 16;   // steps per chunk: two checkpoint intervals
 // Wavefronts per workgroup (independent of each other): four land on the four SIMDs of a compute
 // unit, where single-wavefront workgroups leave some SIMDs with two wavefronts and others with none.
-constexpr int kSplitWaves = 4;   // steps per chunk: two checkpoint intervals
+constexpr int kSplitWaves = 4;
 
 // value of the other lane of the pair (quad_perm [1,0,3,2])
 __device__ __forceinline__ float pair_swap(float v) {
@@ -105,7 +105,7 @@ forward_scan_split(const FwdParams p) {
     const float knb = kNegLog2e * p.bias[role * Dp + j];
     const float m = p.mask_c ? p.mask_c[col] : 1.0f;
     const float sa = (SKIP == 1 && role == 1 && p.scale_x) ? *p.scale_x : 1.0f;   // scale of operand A (x * scale_x)
-    float cur = p.c0[col];
+    float cur = p.c0 ? p.c0[col] : 0.0f;   // no initial state given: zeros
 
     const int64_t L = p.L;
     const int64_t ef = (flip ? (L - 1) : 0) * p.ncols + colu;
@@ -264,7 +264,7 @@ backward_scan_split(const BwdParams p) {
     // scale of operand A: role 1's skip operand is x * scale_x, U[..., 3], or nothing (times zero)
     const float sa = role ? (SKIP == 0 ? 0.0f : sx) : 1.0f;
     const float oa_a = role ? m * sx : 1.0f, oa_b = role ? sx : 1.0f;   // see out_a below (sx is 1 unless the skip term is x)
-    float cur = p.glast[col];   // d loss / d state (meaningful in role 0)
+    float cur = p.glast ? p.glast[col] : 0.0f;   // d loss / d state (meaningful in role 0); not given: zeros
     CompensatedSum sw, sb;      // the lane's gate: sums of its weight_c and bias gradients
 
     const int64_t L = p.L;
@@ -309,8 +309,10 @@ backward_scan_split(const BwdParams p) {
         T1::template load<NTL>(s.gh, ghbase + e0 * 2, off1);
         if (HAS_PAD) s.pad = p.pad[pf + (ch * TC + min(lane % TC, rows - 1)) * ps];
         // one load from a selected address, so that every chunk issues the same operations
-        const float *from = (ch == 0) ? p.c0 + col : p.ckpt + (ch * kRowsPerChunk - 1) * p.ncols + col;
-        s.cstart = *from;
+        // (without an initial state chunk 0 starts from zero: its load reads checkpoint row 0 and drops the value)
+        const float *from = (ch == 0) ? (p.c0 ? p.c0 + col : p.ckpt + col) : p.ckpt + (ch * kRowsPerChunk - 1) * p.ncols + col;
+        const float v = *from;
+        s.cstart = (ch == 0 && !p.c0) ? 0.0f : v;
     };
 
     auto stage_to_lds = [&](const Stage &s) __attribute__((always_inline)) {

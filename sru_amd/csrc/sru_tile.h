@@ -92,46 +92,6 @@ struct RowTile {
         for (int i = 0; i < kPieces; ++i)
             r.v[i] = *reinterpret_cast<const piece_a *>(lds + row_of(i, lane) * PITCH + within(i, lane));
     }
-    // column `lane`'s N elements of row `row`, as floats
-    template <typename T>
-    __device__ __forceinline__ static void read_column(const unsigned char *lds, int row, int lane, float (&out)[N]) {
-        const unsigned char *rowp = lds + row * kRowBytes;
-        if constexpr (N == 1) {
-            out[0] = bits_to_float<T>(reinterpret_cast<const u16_a *>(rowp)[lane]);
-        } else if constexpr (N == 4) {
-            const u32x2_a d = reinterpret_cast<const u32x2_a *>(rowp)[lane];
-            out[0] = bits_to_float<T>(d.x & 0xffffu);
-            out[1] = bits_to_float<T>(d.x >> 16);
-            out[2] = bits_to_float<T>(d.y & 0xffffu);
-            out[3] = bits_to_float<T>(d.y >> 16);
-        } else {
-            static_assert(N == 3, "1, 3 or 4 elements per column");
-            // 6 bytes starting at byte 6 * lane: the two dwords around them, shifted by half a
-            // dword in odd lanes
-            const int first = (3 * lane) >> 1;
-            const uint32_t d0 = reinterpret_cast<const u32_a *>(rowp)[first];
-            const uint32_t d1 = reinterpret_cast<const u32_a *>(rowp)[first + 1];
-            const uint32_t sh = 16u * (uint32_t)(lane & 1);
-            const uint32_t lo = __builtin_amdgcn_alignbit(d1, d0, sh), hi = d1 >> sh;
-            out[0] = bits_to_float<T>(lo & 0xffffu);
-            out[1] = bits_to_float<T>(lo >> 16);
-            out[2] = bits_to_float<T>(hi & 0xffffu);
-        }
-    }
-    template <typename T>
-    __device__ __forceinline__ static void write_column(unsigned char *lds, int row, int lane, const float (&v)[N]) {
-        unsigned char *rowp = lds + row * kRowBytes;
-        if constexpr (N == 4) {
-            u32x2_a d;
-            d.x = pack_pair<T>(v[0], v[1]);
-            d.y = pack_pair<T>(v[2], v[3]);
-            reinterpret_cast<u32x2_a *>(rowp)[lane] = d;
-        } else {
-#pragma unroll
-            for (int i = 0; i < N; ++i)
-                reinterpret_cast<u16_a *>(rowp)[lane * N + i] = (uint16_t)float_to_bits<T>(v[i]);
-        }
-    }
 };
 
 }  // namespace sru_amd

@@ -21,6 +21,7 @@ The large streams (U, x, h, c and their gradients) are consumed in the dtype of
 from typing import Optional, Tuple
 
 import ctypes
+import functools
 
 import torch
 from torch import Tensor
@@ -50,49 +51,66 @@ def _f32(t: Optional[Tensor]) -> Optional[Tensor]:
 
 
 class _Problem:
-    """Sizes and flags derived the way sru/cuda_functional.py:54-65 derives them."""
+    """Sizes and flags derived the way sru/cuda_functional.py:54-65 derives them. Instances are
+    immutable and shared: `_problem()` keeps one per distinct (shape, dtype, flags)."""
 
-    def __init__(self, u: Tensor, x: Tensor, weight_c: Tensor, d_out: int,
-                 bidirectional: bool, has_skip_term: bool, activation_type: int,
-                 checkpoint_state: bool = False):
-        if u.dtype not in _DTYPES:
-            raise ValueError(f"U must be float32, float16 or bfloat16, not {u.dtype}")
-        if not u.is_cuda:
-            raise RuntimeError("the SRU recurrence kernels need device tensors (got a CPU tensor)")
-        if x.dim() not in (2, 3):
+    def __init__(self, dtype, x_dim, length, batch, u_numel, u_last, is_custom, d_out,
+                 bidirectional, has_skip_term, activation_type, checkpoint_state):
+        if dtype not in _DTYPES:
+            raise ValueError(f"U must be float32, float16 or bfloat16, not {dtype}")
+        if x_dim not in (2, 3):
             raise ValueError("x must be 2 or 3 dimensional")
-        self.batch = x.size(-2)
+        self.batch = batch
         self.d = d_out
-        self.length = x.size(0) if x.dim() == 3 else 1
+        self.length = length
         self.dirs = 2 if bidirectional else 1
-        k = u.size(-1) // d_out
+        k = u_last // d_out
         self.k = k // 2 if bidirectional else k
         self.Dp = d_out * self.dirs
-        if u.numel() != self.length * self.batch * self.Dp * self.k:
-            raise ValueError(f"U has {u.numel()} elements, expected length*batch*{self.Dp}*{self.k}")
-        self.is_custom = 1 if weight_c.dim() > 1 else 0
+        if u_numel != self.length * self.batch * self.Dp * self.k:
+            raise ValueError(f"U has {u_numel} elements, expected length*batch*{self.Dp}*{self.k}")
+        self.is_custom = is_custom
         self.skip_type = 0 if not has_skip_term else (1 if self.k == 3 else 2)
         self.activation_type = activation_type
-        self.dtype = u.dtype
-        self.squeeze = x.dim() == 2
+        self.dtype = dtype
+        self.squeeze = x_dim == 2
         # Between forward and backward keep float checkpoints of the state instead of the
         # state after every step wherever the kernels support it (with four streams, a skip
         # term): the backward kernel rebuilds what lies in between.
         # 16-bit streams need an even d for that; a per-step weight_c must not come with tanh.
-        ok = (u.dtype == torch.float32 or d_out % 2 == 0) and not (self.is_custom and activation_type != 0)
+        ok = (dtype == torch.float32 or d_out % 2 == 0) and not (self.is_custom and activation_type != 0)
         self.checkpointed = bool(checkpoint_state and ok and not (self.skip_type == 0 and self.k == 4))
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
                                 activation_type, self.skip_type, self.is_custom,
-                                _DTYPES[u.dtype],
+                                _DTYPES[dtype],
                                 _lib.STATE_INTERVAL if self.checkpointed else 1)
+        lib = _lib.load()
+        self.state_rows = lib.sru_amd_state_bytes(ctypes.byref(self.shape)) // (4 * self.batch * self.Dp) \
+            if self.checkpointed else self.length
+        self.workspace_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(self.shape))
 
     def group_bytes(self):
         es = 4 if self.dtype == torch.float32 else 2
         return es * (4 if self.k == 4 else 1)
 
 
+_problem_cached = functools.lru_cache(maxsize=256)(_Problem)
+
+
+def _problem(u: Tensor, x: Tensor, weight_c: Tensor, d_out: int, bidirectional: bool,
+             has_skip_term: bool, activation_type: int, checkpoint_state: bool = False) -> _Problem:
+    if not u.is_cuda:
+        raise RuntimeError("the SRU recurrence kernels need device tensors (got a CPU tensor)")
+    if x.dim() not in (2, 3):
+        raise ValueError("x must be 2 or 3 dimensional")
+    return _problem_cached(u.dtype, x.dim(), x.size(0) if x.dim() == 3 else 1, x.size(-2), u.numel(),
+                           u.size(-1), 1 if weight_c.dim() > 1 else 0, d_out, bool(bidirectional),
+                           bool(has_skip_term), int(activation_type), bool(checkpoint_state))
+
+
 def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad):
-    u_ = _aligned(u, max(4, pb.group_bytes()))
+    # (16-bit k=4 groups of two columns move as one 16-byte vector in the checkpointed kernels)
+    u_ = _aligned(u, 16)
     x_ = None
     if pb.skip_type == 1:
         x_ = _aligned(x if x.dtype == pb.dtype else x.to(pb.dtype), 4)
@@ -107,8 +125,8 @@ def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, m
         if wc_.numel() != 2 * pb.Dp:
             raise ValueError("weight_c must have 2*output_size elements")
     bias_ = _f32(bias)
-    init_ = _f32(init)
-    if bias_.numel() != 2 * pb.Dp or init_.numel() != pb.batch * pb.Dp:
+    init_ = _f32(init)         # None: the kernels start from zeros
+    if bias_.numel() != 2 * pb.Dp or (init_ is not None and init_.numel() != pb.batch * pb.Dp):
         raise ValueError("bias must have 2*output_size and init batch*output_size elements")
     mask_c_ = _f32(mask_c)
     if mask_c_ is not None and mask_c_.numel() != pb.batch * pb.Dp:
@@ -132,8 +150,7 @@ def _run_forward(pb, u_, x_, wc_, bias_, init_, scale_, mask_c_, pad_, keep_c: b
     h = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
     c = None
     if keep_c and pb.checkpointed:
-        rows = lib.sru_amd_state_bytes(ctypes.byref(pb.shape)) // (4 * pb.batch * pb.Dp)
-        c = torch.empty(rows, pb.batch, pb.Dp, dtype=torch.float32, device=dev)
+        c = torch.empty(pb.state_rows, pb.batch, pb.Dp, dtype=torch.float32, device=dev)
     elif keep_c:
         c = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
     c_last = torch.empty(pb.batch, pb.Dp, dtype=torch.float32, device=dev)
@@ -146,21 +163,35 @@ def _run_forward(pb, u_, x_, wc_, bias_, init_, scale_, mask_c_, pad_, keep_c: b
     return h, c, c_last
 
 
+def _kernel_dtype(u: Tensor) -> torch.dtype:
+    """Stream dtype the kernels run in for a U of this dtype: float16 and bfloat16 as they are,
+    everything else float32 (float64 included: the reference's training entry casts it to float32
+    as well, sru/ops.py:116-127)."""
+    return u.dtype if u.dtype in (torch.float16, torch.bfloat16) else torch.float32
+
+
 def elementwise_recurrence_forward(
-        u: Tensor, x: Tensor, weight_c: Tensor, bias: Tensor, init: Tensor,
+        u: Tensor, x: Tensor, weight_c: Tensor, bias: Tensor, init: Optional[Tensor],
         activation_type: int, d_out: int, bidirectional: bool, has_skip_term: bool,
         scale_x: Optional[Tensor] = None, mask_c: Optional[Tensor] = None,
         mask_pad: Optional[Tensor] = None, keep_c: bool = True
 ) -> Tuple[Tensor, Tensor, Optional[Tensor]]:
-    """Forward scan; returns (h, last_hidden, c) as sru/cuda_functional.py:37-153 does.
+    """Forward scan; returns (h, last_hidden, c) as sru/cuda_functional.py:37-153 does, in U's dtype.
 
     `keep_c=False` (no counterpart in the reference) skips storing the per-step
-    state and returns None for it: the inference variant.
+    state and returns None for it: the inference variant. `init=None` stands for zeros.
+    A float64 U is computed in float32 and the results are cast back.
     """
-    pb = _Problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type)
+    out_dtype = u.dtype
+    if u.dtype != _kernel_dtype(u):
+        u = u.to(_kernel_dtype(u))
+    pb = _problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type)
     prepared = _prepare_inputs(pb, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad)
     h, c, c_last = _run_forward(pb, *prepared, keep_c=keep_c)
-    last_hidden = c_last if pb.dtype == torch.float32 else c_last.to(pb.dtype)
+    last_hidden = c_last if out_dtype == torch.float32 else c_last.to(out_dtype)
+    if out_dtype != pb.dtype:
+        h = h.to(out_dtype)
+        c = c.to(out_dtype) if c is not None else None
     if pb.squeeze:
         h = h.squeeze(0)
         c = c.squeeze(0) if c is not None else None
@@ -168,21 +199,33 @@ def elementwise_recurrence_forward(
 
 
 class ElementwiseRecurrence(Function):
-    """Drop-in for sru/cuda_functional.py:156-261."""
+    """Drop-in for sru/cuda_functional.py:156-261.
+
+    Beyond the reference's argument list: `init` may be None (zeros, and no gradient for it). A
+    float64 U (which the reference's kernels compute in double) is computed in float32 here; outputs
+    and gradients come back in the dtypes of the inputs."""
 
     @staticmethod
     def forward(ctx, u, x, weight_c, bias, init, activation_type, d_out, bidirectional,
                 has_skip_term, scale_x, mask_c=None, mask_pad=None):
-        pb = _Problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type,
+        # gradients that autograd does not have stay None instead of becoming zero tensors (one
+        # fill kernel per layer for the usually unused gradient of the last state)
+        ctx.set_materialize_grads(False)
+        u_dtype = u.dtype
+        if u.dtype != _kernel_dtype(u):
+            u = u.to(_kernel_dtype(u))
+        pb = _problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type,
                       checkpoint_state=True)
         prepared = _prepare_inputs(pb, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad)
         h, c, c_last = _run_forward(pb, *prepared, keep_c=True)
         ctx.problem = pb
-        ctx.in_dtypes = (x.dtype, weight_c.dtype, bias.dtype, init.dtype)
-        ctx.in_shapes = (u.shape, x.shape, weight_c.shape, bias.shape, init.shape)
+        ctx.in_dtypes = (u_dtype, x.dtype, weight_c.dtype, bias.dtype, None if init is None else init.dtype)
+        ctx.in_shapes = (u.shape, x.shape, weight_c.shape, bias.shape, None if init is None else init.shape)
         ctx.save_for_backward(*[t for t in prepared if t is not None], c)
         ctx.present = [t is not None for t in prepared]
-        last_hidden = c_last if pb.dtype == torch.float32 else c_last.to(pb.dtype)
+        last_hidden = c_last if u_dtype == torch.float32 else c_last.to(u_dtype)
+        if u_dtype != pb.dtype:
+            h = h.to(u_dtype)
         if pb.squeeze:
             h = h.squeeze(0)
         return h, last_hidden
@@ -195,32 +238,35 @@ class ElementwiseRecurrence(Function):
         it = iter(saved)
         u_, x_, wc_, bias_, init_, scale_, mask_c_, pad_ = [next(it) if p else None for p in ctx.present]
         dev = u_.device
-        gh = _aligned(grad_h if grad_h.dtype == pb.dtype else grad_h.to(pb.dtype), 4)
-        gl = _f32(grad_last)
+        if grad_h is None:     # only last_hidden was used downstream
+            gh = torch.zeros(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
+        else:
+            gh = _aligned(grad_h if grad_h.dtype == pb.dtype else grad_h.to(pb.dtype), 4)
+        gl = _f32(grad_last)   # None: the kernels start from a zero state gradient
         grad_u = torch.empty_like(u_)
         grad_x = torch.empty_like(x_) if pb.skip_type == 1 else None
         grad_wc = torch.empty_like(wc_) if pb.is_custom else \
             torch.empty(2 * pb.Dp, dtype=torch.float32, device=dev)
-        grad_bias = torch.empty(2 * pb.Dp, dtype=torch.float32, device=dev)
-        grad_init = torch.empty(pb.batch, pb.Dp, dtype=torch.float32, device=dev)
-        lib = _lib.load()
-        ws_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(pb.shape))
+        # grad_bias (2, D') and grad_init (B, D') share one allocation
+        small = torch.empty((2 + pb.batch) * pb.Dp, dtype=torch.float32, device=dev)
+        grad_bias, grad_init = small[:2 * pb.Dp], small[2 * pb.Dp:]
+        ws_bytes = pb.workspace_bytes
         workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
         with torch.cuda.device(dev):
             stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-            rc = lib.sru_amd_backward(
+            rc = _lib.load().sru_amd_backward(
                 ctypes.byref(pb.shape), _ptr(u_), _ptr(x_), _ptr(wc_), _ptr(bias_), _ptr(init_),
                 _ptr(mask_c_), _ptr(pad_), _ptr(scale_), _ptr(c), _ptr(gh), _ptr(gl),
                 _ptr(grad_u), _ptr(grad_x), _ptr(grad_wc), _ptr(grad_bias), _ptr(grad_init),
                 _ptr(workspace), ctypes.c_size_t(ws_bytes), stream)
         _lib.check(rc, "sru_amd_backward")
-        x_dt, wc_dt, bias_dt, init_dt = ctx.in_dtypes
+        u_dt, x_dt, wc_dt, bias_dt, init_dt = ctx.in_dtypes
         u_sh, x_sh, wc_sh, bias_sh, init_sh = ctx.in_shapes
-        grad_u = grad_u.view(u_sh)
+        grad_u = grad_u.view(u_sh).to(u_dt)
         if grad_x is not None:
             grad_x = grad_x.view(x_sh).to(x_dt)
         grad_wc = grad_wc.view(wc_sh).to(wc_dt)
         grad_bias = grad_bias.view(bias_sh).to(bias_dt)
-        grad_init = grad_init.view(init_sh).to(init_dt)
+        grad_init = None if init_sh is None else grad_init.view(init_sh).to(init_dt)
         return grad_u, grad_x, grad_wc, grad_bias, grad_init, \
             None, None, None, None, None, None, None

@@ -127,8 +127,8 @@ class SRUCell(nn.Module):
         if input.dim() not in (2, 3):
             raise ValueError("Input must be 2 or 3 dimensional")
         batch = input.size(-2)
-        if c0 is None:
-            c0 = torch.zeros(batch, self.output_size, dtype=input.dtype, device=input.device)
+        # (c0 = None goes down to the kernels as it is: they start from zeros, and no zero tensor is
+        # allocated and filled per layer as at sru/modules.py:241-243)
 
         residual = input                                   # the skip term is the un-normalised input
         if self.layer_norm is not None and not self.normalize_after:
@@ -155,11 +155,14 @@ class SRUCell(nn.Module):
         if not fused_layer_norm_supported(x) or ln.weight is None or ln.bias is None:
             return ln(x)
         out_dtype = x.dtype
-        if feeds_projection and torch.is_autocast_enabled("cuda"):
+        # (only when the dense product is the direct consumer: a custom module or the rnn_dropout
+        # multiply in between sees what nn.LayerNorm would have given them, rows in x's dtype)
+        direct = self.custom_m is None and not (self.training and self.rnn_dropout > 0)
+        if feeds_projection and direct and torch.is_autocast_enabled("cuda"):
             out_dtype = torch.get_autocast_dtype("cuda")
         return fused_layer_norm(x, ln.weight, ln.bias, ln.eps, out_dtype)
 
-    def apply_recurrence(self, U: Tensor, V: Tensor, residual: Tensor, c0: Tensor,
+    def apply_recurrence(self, U: Tensor, V: Tensor, residual: Tensor, c0: Optional[Tensor],
                          scale_val: Optional[Tensor], mask_c: Optional[Tensor],
                          mask_pad: Optional[Tensor]) -> List[Tensor]:
         """The call of sru/modules.py:296-304: always the training entry, which itself skips the
@@ -297,8 +300,7 @@ class SRU(nn.Module):
         if input.dim() != 3:
             raise ValueError("There must be 3 dimensions for (length, batch_size, input_size)")
         if c0 is None:
-            zeros = torch.zeros(input.size(1), self.output_size, dtype=input.dtype, device=input.device)
-            states = [zeros] * self.num_layers
+            states = [None] * self.num_layers      # the kernels start from zeros (sru/modules.py:617-620)
         else:
             if c0.dim() != 3:
                 raise ValueError("c0 must be 3 dim (num_layers, batch_size, output_size)")

@@ -6,9 +6,10 @@ normalised rows leave the kernel already in the 16-bit dtype the projection cons
 HIP kernels of csrc/sru_norm.hip through the C ABI (include/sru_amd.h); `supported()` says whether
 a tensor can take that path (device tensor, feature count a multiple of 8 and at most
 SRU_AMD_NORM_MAX_FEATURES) - anything else is torch's own layer_norm, which is the operation the
-reference itself calls.
+reference itself calls; `layer_norm` says so with a warning (or raises with `strict=True`).
 """
 import ctypes
+import warnings
 from typing import Optional
 
 import torch
@@ -66,13 +67,27 @@ class LayerNormFunction(Function):
         return grad_x, grad_wb[0].to(wdt), grad_wb[1].to(bdt), None, None
 
 
+_warned_widths = set()
+
+
 def layer_norm(x: Tensor, weight: Tensor, bias: Tensor, eps: float = 1e-5,
-               out_dtype: Optional[torch.dtype] = None) -> Tensor:
-    """Normalises over the last dimension; `out_dtype` defaults to x's dtype."""
+               out_dtype: Optional[torch.dtype] = None, strict: bool = False) -> Tensor:
+    """Normalises over the last dimension; `out_dtype` defaults to x's dtype.
+
+    A tensor the kernels do not take (see `supported`) goes through torch's own layer_norm, once
+    per feature count with a warning; `strict=True` raises instead."""
     out_dtype = out_dtype or x.dtype
     if out_dtype not in _DTYPES:
         raise ValueError(f"out_dtype must be float32, float16 or bfloat16, not {out_dtype}")
     if not supported(x):
+        why = (f"sru_amd.norm.layer_norm: no kernel for a {x.dtype} {'device' if x.is_cuda else 'CPU'} tensor with "
+               f"{x.size(-1)} features (needs a device tensor, a multiple of 8 and at most {_lib.NORM_MAX_FEATURES})")
+        if strict:
+            raise ValueError(why)
+        key = (x.size(-1), x.dtype, x.is_cuda)
+        if key not in _warned_widths:
+            _warned_widths.add(key)
+            warnings.warn(why + "; using torch.nn.functional.layer_norm")
         y = torch.nn.functional.layer_norm(x.float(), (x.size(-1),), weight.float(), bias.float(), eps)
         return y.to(out_dtype)
     return LayerNormFunction.apply(x, weight, bias, eps, out_dtype)

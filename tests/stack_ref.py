@@ -92,11 +92,12 @@ def record_dropout_masks(model):
     return undo
 
 
-def stack_forward_large(model, x, mask_pad=None, masks=None, device="cuda:0"):
+def stack_forward_large(model, x, mask_pad=None, masks=None, device="cuda:0", c0=None):
     """Float64 restatement of a whole stack at sizes where stack_forward is too slow: the dense
     products run in float64 on `device` (torch), the recurrence in the C oracle on the host.
     `masks`: per layer, the mask_c that layer drew in the run being checked (None = eval mode;
-    rnn_dropout is not supported). Returns (h, c_stack, params) like stack_forward."""
+    rnn_dropout is not supported). `c0`: (layers, B, D') initial states or None for zeros.
+    Returns (h, c_stack, params) like stack_forward."""
     dt = torch.float64
     params = {n: p.detach().to(device, dt).requires_grad_(True) for n, p in model.named_parameters()}
     x = x.detach().to(device, dt)
@@ -114,7 +115,8 @@ def stack_forward_large(model, x, mask_pad=None, masks=None, device="cuda:0"):
         if cell.projection_size:
             flat = flat @ g("weight_proj")
         U = (flat @ g("weight")).reshape(L, B, -1)
-        init = torch.zeros(B, cell.output_size, dtype=dt, device=device)
+        init = torch.zeros(B, cell.output_size, dtype=dt, device=device) if c0 is None \
+            else c0[i].detach().to(device, dt)
         scale = float(cell.scale_x.item()) if cell.rescale else None
         mask_c = None if masks is None or masks[i] is None else masks[i].detach().to(device, dt)
         h, c = OracleRecurrence.apply(U, residual, g("weight_c"), g("bias"), init, cell.activation_type,

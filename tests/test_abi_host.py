@@ -61,7 +61,7 @@ def test_null_and_misaligned_pointers_and_workspace():
     s = _shape()
     assert lib.sru_amd_forward(None, *([FAKE] * 11), None) == 1
     args = [FAKE] * 11
-    for required in (0, 1, 2, 3, 4, 8, 10):   # u, x (skip from x), weight_c, bias, c_init, h, c_last
+    for required in (0, 1, 2, 3, 8, 10):   # u, x (skip from x), weight_c, bias, h, c_last (c_init may be NULL: zeros)
         bad = list(args)
         bad[required] = None
         assert lib.sru_amd_forward(ctypes.byref(s), *bad, None) == 1, required
@@ -81,9 +81,12 @@ def test_null_and_misaligned_pointers_and_workspace():
     assert lib.sru_amd_state_bytes(ctypes.byref(_shape(length=33, state_interval=8, dtype=1))) == 4 * 2 * 16 * 4
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 16), None, need, None) == 6
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), need - 1, None) == 6
-    bad = [FAKE] * 17
-    bad[13] = None                               # grad_x is required when the skip term is x
-    assert lib.sru_amd_backward(ctypes.byref(s), *bad, need, None) == 1
+    # u, x, weight_c, bias, c, grad_h, grad_u, grad_x, grad_wc, grad_bias, grad_init
+    # (c_init = 4 and grad_last = 10 may be NULL: zeros)
+    for required in (0, 1, 2, 3, 8, 9, 11, 12, 13, 14, 15):
+        bad = [FAKE] * 17                        # e.g. 12: grad_x is required when the skip term is x
+        bad[required] = None
+        assert lib.sru_amd_backward(ctypes.byref(s), *bad, need, None) == 1, required
 
 
 def test_static_backward_checks_sizes_before_anything_else():

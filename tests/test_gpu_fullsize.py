@@ -215,7 +215,7 @@ def test_offsets_beyond_32_bits_long_sequence_k4():
     assert not torch.isnan(h_big[-1]).any() and not torch.isnan(h_big[0]).any()
     rows = torch.tensor([0, B - 1], device=dev)
     h_small, cl_small = run(U[:, rows].contiguous(), c0[rows].contiguous(), pad[:, rows], 2)
-    # the two runs select different kernels (two columns per lane for the wide one, row tiles for
+    # the two runs select different kernels (two columns per lane for the wide one, lane pairs for
     # the narrow one) whose float arithmetic is the same up to the compiler's choice of fused
     # multiply-adds: the final states agree to 1e-6, the float16 outputs to one unit in the last place
     a, b = h_big[:, rows].float(), h_small.float()
@@ -223,6 +223,66 @@ def test_offsets_beyond_32_bits_long_sequence_k4():
     assert float((a != b).float().mean()) <= 1e-3
     assert float((cl_big[rows] - cl_small).abs().max()) <= 1e-6 * max(1.0, float(cl_small.abs().max()))
     assert float(h_big[pad].abs().max()) == 0.0
+
+
+def test_long_sequence_inference_full_size_k3_fp16():
+    """The long-sequence inference workload at its real size: bidirectional, d=256, L=4096, B=256,
+    float16 streams, k=3 with the skip term read from x, lengths in [1024, 4096], c0 ~ N(0,1), state
+    not stored. Inputs are drawn on the device (as float64 host arrays they would not fit). Checked
+    three ways: padded cells are zero; the first and the last batch row equal a run on those two rows
+    alone (another kernel: the lane-pair one); and those two rows equal the float64 oracle fed the
+    same rounded values."""
+    import ctypes
+    from sru_amd import _lib
+    L, B, d, dirs, k = 4096, 256, 256, 2, 3
+    Dp = d * dirs
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(78)
+    U = torch.empty(L, B, Dp * k, dtype=torch.float16, device=dev)
+    x = torch.empty(L, B, Dp, dtype=torch.float16, device=dev)
+    for t0 in range(0, L, 512):
+        U[t0:t0 + 512] = torch.randn(512, B, Dp * k, device=dev, generator=g).half()
+        x[t0:t0 + 512] = torch.randn(512, B, Dp, device=dev, generator=g).half()
+    wc = (torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1)
+    bias = torch.randn(2 * Dp, device=dev, generator=g) * 0.3
+    c0 = torch.randn(B, Dp, device=dev, generator=g)
+    scale = torch.tensor([1.7], device=dev)
+    lens = torch.randint(1024, L + 1, (B,), device=dev, generator=g)
+    lens[0], lens[B - 1] = L, 1024          # the two rows looked at closely: the longest and the shortest
+    pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :])
+    lib = _lib.load()
+    p = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+
+    def run(U_, x_, c0_, pad_, batch):
+        shape = _lib.Shape(L, batch, d, dirs, k, 0, 1, 0, _lib.F16, 1)
+        h = torch.full((L, batch, Dp), float("nan"), dtype=torch.float16, device=dev)
+        cl = torch.full((batch, Dp), float("nan"), device=dev)
+        padb = pad_.contiguous().view(torch.uint8)
+        rc = lib.sru_amd_forward(ctypes.byref(shape), p(U_), p(x_), p(wc), p(bias), p(c0_), None, p(padb),
+                                 p(scale), p(h), None, p(cl), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, _lib.status_string(rc)
+        torch.cuda.synchronize()
+        return h, cl
+
+    h_big, cl_big = run(U, x, c0, pad, B)
+    assert not torch.isnan(h_big).any() and not torch.isnan(cl_big).any()
+    assert float(h_big[pad].abs().max()) == 0.0
+    rows = torch.tensor([0, B - 1], device=dev)
+    U2, x2, c02, pad2 = U[:, rows].contiguous(), x[:, rows].contiguous(), c0[rows].contiguous(), pad[:, rows]
+    h_small, cl_small = run(U2, x2, c02, pad2, 2)
+    # two kernels whose float arithmetic agrees up to the compiler's choice of fused multiply-adds:
+    # final states to 1e-6, float16 outputs to one unit in the last place in a few cells
+    a, b = h_big[:, rows].float(), h_small.float()
+    assert float(((a - b).abs() / b.abs().clamp(min=1.0)).max()) <= 2.0 ** -10
+    assert float((a != b).float().mean()) <= 5e-3
+    assert float((cl_big[rows] - cl_small).abs().max()) <= 1e-6 * max(1.0, float(cl_small.abs().max()))
+    # the same two rows against the float64 oracle
+    n = lambda t: t.double().cpu().numpy()
+    h_ref, _, cl_ref = so.forward(n(U2), n(x2), n(wc), n(bias), n(c02), d=d, dirs=dirs, k=k, activation_type=0,
+                                  skip_type=1, is_custom=0, scale_x=float(scale.item()), mask_c=None,
+                                  mask_pad=pad2.cpu().numpy())
+    assert _maxerr(n(h_big[:, rows]), h_ref) <= 2e-2 * max(1.0, np.abs(h_ref).max())
+    assert _maxerr(n(cl_big[rows]), cl_ref) <= 1e-3 * max(1.0, np.abs(cl_ref).max())
 
 
 @pytest.mark.parametrize("checkpointed", [False, True], ids=["state_every_step", "state_checkpoints"])

@@ -86,3 +86,76 @@ def test_amp_style_bf16_streams_against_fp32_run():
         outs[native] = [h.float()] + [v.grad.float() for v in (u, x, wc, bias, c0)]
     for a, b in zip(outs[True], outs[False]):
         assert float((a - b).detach().abs().max()) <= 2e-2 * max(1.0, float(b.detach().abs().max()))
+
+
+def test_float64_inputs_are_computed_in_float32_and_come_back_as_given():
+    # the reference's training entry casts float64 to float32 and returns float32 (sru/ops.py:116-127);
+    # its autograd Function, called directly, keeps the dtype of U (its kernels exist for double,
+    # sru/csrc/sru_cuda_kernel.cu:845). Here both compute in float32.
+    from sru_amd import ElementwiseRecurrence, elementwise_recurrence_gpu
+    c = Case(L=14, B=3, d=64, dirs=2, seed=44, pad="right", scale=1.7, mask_c=True).f32()
+    h64, last64, g64 = _apply(ElementwiseRecurrence.apply, c, "cuda:0", torch.float64)
+    h_ref, last_ref, g_ref = _apply(st.recurrence, c, "cpu", torch.float64)
+    assert np.abs(h64 - h_ref).max() <= 1e-5 and np.abs(last64 - last_ref).max() <= 1e-5
+    for a, b in zip(g64, g_ref):
+        assert a is not None and np.abs(a - b).max() <= 1e-5 * max(1.0, np.abs(b).max())
+    dev = "cuda:0"
+    t = lambda a: torch.tensor(a, dtype=torch.float64, device=dev, requires_grad=True)
+    u, x, wc, bias, c0 = t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0)
+    h, last = ElementwiseRecurrence.apply(u, x, wc, bias, c0, 0, c.d, True, True, None, None, None)
+    assert h.dtype == torch.float64 and last.dtype == torch.float64
+    h.sum().backward()
+    assert all(v.grad is not None and v.grad.dtype == torch.float64 for v in (u, x, wc, bias, c0))
+    h, last = elementwise_recurrence_gpu(u, x, wc, bias, c0, 0, c.d, True, True)
+    assert h.dtype == torch.float32 and last.dtype == torch.float32
+    with torch.no_grad():
+        h, last = elementwise_recurrence_gpu(u, x, wc, bias, c0, 0, c.d, True, True)
+    assert h.dtype == torch.float32
+
+
+def test_no_initial_state_no_last_state_gradient_and_last_state_only():
+    # init = None stands for zeros (no zero tensor is built); a loss that does not use last_hidden
+    # hands the backward kernel no grad_last; a loss that uses only last_hidden hands it no grad_h
+    from sru_amd import ElementwiseRecurrence
+    c = Case(L=21, B=3, d=64, dirs=2, seed=45, scale=1.3, zero_c0=True).f32()
+    dev = "cuda:0"
+    t = lambda a: torch.tensor(a, dtype=torch.float32, device=dev, requires_grad=True)
+    sx = torch.tensor([c.scale], device=dev)
+    gh = torch.tensor(c.gh, dtype=torch.float32, device=dev)
+    gl = torch.tensor(c.gl, dtype=torch.float32, device=dev)
+    results = {}
+    for name, init_none, loss in (("zeros", False, "both"), ("none", True, "both"), ("h_only", True, "h"),
+                                  ("h_only_ref", False, "h"), ("last_only", True, "last"), ("last_only_ref", False, "last")):
+        u, x, wc, bias = t(c.U), t(c.x), t(c.wc), t(c.bias)
+        c0 = None if init_none else t(c.c0)
+        h, last = ElementwiseRecurrence.apply(u, x, wc, bias, c0, 0, c.d, True, True, sx, None, None)
+        total = 0
+        if loss in ("both", "h"):
+            total = total + (h * gh).sum()
+        if loss in ("both", "last"):
+            total = total + (last * gl).sum()
+        total.backward()
+        results[name] = [h.detach(), last.detach()] + [v.grad for v in (u, x, wc, bias)]
+    for a, b in (("none", "zeros"), ("h_only", "h_only_ref"), ("last_only", "last_only_ref")):
+        for got, ref in zip(results[a], results[b]):
+            assert torch.equal(got, ref), (a, b)
+
+
+def test_u_view_at_an_unaligned_offset_is_copied_not_refused():
+    # a contiguous U whose storage offset is 8 bytes: the 16-bit k=4 checkpoint kernels need 16
+    from sru_amd import ElementwiseRecurrence
+    c = Case(L=16, B=2, d=64, dirs=2, k=4, seed=46)
+    dev = "cuda:0"
+    flat = torch.zeros(c.U.size + 4, dtype=torch.bfloat16, device=dev)
+    flat[4:] = torch.tensor(c.U, dtype=torch.bfloat16, device=dev).reshape(-1)
+    u_view = flat[4:].view(c.L, c.B, -1).requires_grad_(True)
+    assert u_view.data_ptr() % 16 == 8 and u_view.is_contiguous()
+    u_own = u_view.detach().clone().requires_grad_(True)
+    t = lambda a: torch.tensor(a, dtype=torch.float32, device=dev)
+    x = torch.tensor(c.x, dtype=torch.bfloat16, device=dev)
+    outs = []
+    for u in (u_view, u_own):
+        h, last = ElementwiseRecurrence.apply(u, x, t(c.wc), t(c.bias), t(c.c0), 0, c.d, True, True, None, None, None)
+        h.float().sum().backward()
+        outs.append((h.detach(), u.grad))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])

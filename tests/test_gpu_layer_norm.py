@@ -84,7 +84,11 @@ def test_unsupported_shapes_take_torch_layer_norm():
     x = torch.randn(4, 6, 7, device=DEV)          # 7 features: not a multiple of 8
     assert not supported(x) and supported(torch.randn(4, 16, device=DEV))
     w, b = torch.randn(7, device=DEV), torch.randn(7, device=DEV)
-    assert torch.allclose(layer_norm(x, w, b), F.layer_norm(x, (7,), w, b), atol=1e-6)
+    with pytest.warns(UserWarning, match="no kernel for"):       # the second path is never silent
+        y = layer_norm(x, w, b)
+    assert torch.allclose(y, F.layer_norm(x, (7,), w, b), atol=1e-6)
+    with pytest.raises(ValueError, match="no kernel for"):
+        layer_norm(x, w, b, strict=True)
     with pytest.raises(ValueError):
         layer_norm(x, w, b, out_dtype=torch.float64)
 

@@ -232,3 +232,20 @@ def test_training_mode_under_no_grad_uses_the_dropout_mask(amp):
         p.requires_grad_(False)
     h_frozen, _ = run()
     assert torch.equal(h_frozen, h_ng)
+
+
+def test_double_precision_module_runs_in_float32_as_the_reference_does():
+    # a .double() model: the reference's training entry casts to float32 and returns a float32 h
+    # (sru/ops.py:116-127); one layer, because its second layer would multiply that float32 h with
+    # float64 weights and fail (sru/modules.py:363-378), and so it does here
+    torch.manual_seed(7)
+    cell = SRUCell(16, 16, bidirectional=True).to(DEV).double()
+    x = torch.randn(9, 3, 16, device=DEV, dtype=torch.float64, requires_grad=True)
+    h, c = cell(x)
+    assert h.dtype == torch.float32 and c.dtype == torch.float32
+    h.sum().backward()
+    assert x.grad.dtype == torch.float64 and cell.weight.grad.dtype == torch.float64
+    ref = SRU(16, 16, num_layers=1, bidirectional=True).to(DEV)
+    ref.rnn_lst[0].load_state_dict({k: v.float() for k, v in cell.state_dict().items()})
+    h32, _ = ref(x.detach().float())
+    assert float((h - h32).abs().max()) <= 1e-5

@@ -217,8 +217,8 @@ def test_padded_cells_cannot_leak_bit_identical():
 
 @pytest.mark.parametrize("dt,checkpointed", [("f32", False), ("f32", True), ("bf16", True), ("f16", True)])
 def test_backward_is_bit_reproducible(dt, checkpointed):
-    # also: repeated backward calls on one state buffer (the checkpoint kernels count arrivals in
-    # it to add up the batch sums and must leave the counters as they found them)
+    # repeated backward calls on one state buffer: the batch sums are added in a fixed order, and the
+    # backward call leaves the state buffer as it found it
     for cfg in (dict(L=50, B=16, d=256, dirs=2, pad="right"), dict(L=23, B=5, d=96, dirs=1, k=4),
                 dict(L=9, B=1, d=64, dirs=2, mask_c=True)):
         c = Case(seed=35, **cfg)

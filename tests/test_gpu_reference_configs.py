@@ -1,4 +1,4 @@
-"""The deep and the wide reference workloads at their real sizes.
+"""The reference workloads at their real sizes (the long-sequence one at a reduced batch).
 
 * "config 4": language-model-scale stack, 10 unidirectional layers, hidden 2048, projection 512,
   L=512, B=16, bf16 autocast, dropout 0.1 (a per-layer mask_c), inputs = embedding rows N(0, 0.02).
@@ -6,6 +6,14 @@
   the lane-pairing kernels.
 * "config 3": classification-scale stack, 4 bidirectional layers, d=1024, L=256, B=64, layer norm,
   rescale, fp32 and bf16 autocast.
+* "config 1": the README example, 2 unidirectional layers, input = hidden = 128, L=20, B=32, fp32,
+  highway_bias=-2, forward only.
+* "config 2": 4 bidirectional layers, input = hidden = 512, L=128, B=32, fp32, forward + backward,
+  right-padded batch with lengths in [32, 128], loss = sum(h * probe).
+* "config 5": long-sequence inference, 2 bidirectional layers, d=256, L=4096, fp16 weights and
+  inputs, no_grad, lengths in [1024, 4096], c0 ~ N(0,1); batch 16 instead of 256 so that the
+  float64 host oracle finishes in seconds (the one-layer recurrence runs at B=256 in
+  tests/test_gpu_fullsize.py).
 
 Op level: the kernels through the C ABI against the float64 oracle on identical (rounded) inputs.
 Module level: the whole stack against a float64 restatement (dense products in float64 on the
@@ -120,3 +128,58 @@ def test_config_3_stack_with_layer_norm_and_rescale(amp):
         assert eh <= 1e-4 and ec <= 1e-4 and worst <= 1e-3
     else:
         assert eh <= 2e-2 and ec <= 2e-2 and worst <= 3e-2
+
+
+def test_config_1_readme_example_forward():
+    torch.manual_seed(101)
+    model = SRU(128, 128, num_layers=2, highway_bias=-2.0).to(DEV).eval()
+    x = torch.randn(20, 32, 128, device=DEV)
+    with torch.no_grad():
+        h, c = model(x)
+        h_ref, c_ref, _ = stack_forward_large(model, x, device=DEV)
+    eh = float((h.double() - h_ref).abs().max())
+    ec = float((c.double() - c_ref).abs().max())
+    print(f"\nconfig 1 stack (fp32, forward): max abs error h {eh:.3g}, final states {ec:.3g}")
+    assert h.shape == (20, 32, 128) and c.shape == (2, 32, 128)
+    assert eh <= 1e-5 and ec <= 1e-5
+
+
+def test_config_2_stack_padded_batch_forward_and_backward():
+    torch.manual_seed(202)
+    L, B = 128, 32
+    model = SRU(512, 512, num_layers=4, bidirectional=True).to(DEV)
+    x = torch.randn(L, B, 512, device=DEV)
+    lens = torch.randint(32, L + 1, (B,), device=DEV)
+    lens[0] = L
+    mask_pad = torch.arange(L, device=DEV)[:, None] >= lens[None, :]
+    h, c = model(x, mask_pad=mask_pad)
+    probe = torch.randn(h.shape, device=DEV)
+    (h * probe).sum().backward()
+    h_ref, c_ref, params = stack_forward_large(model, x, mask_pad=mask_pad, device=DEV)
+    (h_ref * probe.double()).sum().backward()
+    eh, ec = _rel(h, h_ref), _rel(c, c_ref)
+    worst = max(_rel(p.grad, params[n].grad) for n, p in model.named_parameters())
+    print(f"\nconfig 2 stack (fp32, lengths in [32, 128]): h {eh:.3g}, final states {ec:.3g}, "
+          f"worst parameter gradient {worst:.3g} (max-abs error / max|ref|)")
+    # every layer zeroes its padded outputs
+    assert float(h[mask_pad].abs().max()) == 0.0
+    assert eh <= 1e-5 and ec <= 1e-5 and worst <= 1e-4
+
+
+def test_config_5_stack_long_sequence_fp16_inference():
+    torch.manual_seed(505)
+    L, B = 4096, 16
+    model = SRU(256, 256, num_layers=2, bidirectional=True).to(DEV).half().eval()
+    x = torch.randn(L, B, 256, device=DEV).half()
+    c0 = torch.randn(2, B, 512, device=DEV).half()
+    lens = torch.randint(1024, L + 1, (B,), device=DEV)
+    lens[0] = L
+    mask_pad = torch.arange(L, device=DEV)[:, None] >= lens[None, :]
+    with torch.no_grad():
+        h, c = model(x, c0, mask_pad=mask_pad)
+        h_ref, c_ref, _ = stack_forward_large(model, x, mask_pad=mask_pad, device=DEV, c0=c0)
+    assert h.dtype == torch.float16 and c.dtype == torch.float16
+    eh, ec = _rel(h, h_ref), _rel(c, c_ref)
+    print(f"\nconfig 5 stack (fp16, L=4096, B={B}): h {eh:.3g}, final states {ec:.3g} (max-abs error / max|ref|)")
+    assert float(h[mask_pad].abs().max()) == 0.0
+    assert eh <= 2e-2 and ec <= 2e-2

@@ -146,3 +146,72 @@ def test_two_host_threads_on_two_streams():
     for a, b in zip(alone, together):
         for x, y in zip(a, b):
             assert torch.equal(x, y)
+
+
+def _timed(fn, n=200):
+    import time
+    for _ in range(10):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e6 / n
+
+
+def test_graphed_helper_forward_only_readme_example():
+    """sru_amd.graphed on the README-example stack in eval mode: every replay equals the eager result
+    for the input it is given (with eager work and a sync in between), and a replay is faster than
+    the eager call it replaces (the eager call is all host-side launch work at this size)."""
+    import sru_amd
+    torch.manual_seed(6)
+    model = sru_amd.SRU(128, 128, num_layers=2, highway_bias=-2.0).cuda().eval()
+    x0 = torch.randn(20, 32, 128, device="cuda")
+    with torch.no_grad():
+        fast = sru_amd.graphed(model, x0)
+        assert not fast.training
+        for replay in range(3):
+            x = torch.randn(20, 32, 128, device="cuda")
+            h_eager, c_eager = model(x)
+            torch.cuda.synchronize()
+            h, c = fast(x)
+            torch.cuda.synchronize()
+            assert torch.equal(h, h_eager) and torch.equal(c, c_eager), replay
+        eager_us = _timed(lambda: model(x0))
+        replay_us = _timed(lambda: fast(x0))
+    print(f"\nREADME-example stack, forward: eager {eager_us:.1f} us per call, graph replay {replay_us:.1f} us")
+    assert replay_us < eager_us
+    with pytest.raises(ValueError):
+        fast(torch.randn(21, 32, 128, device="cuda"))
+    with pytest.raises(ValueError):
+        fast(x0, mask_pad=torch.zeros(20, 32, dtype=torch.bool, device="cuda"))
+
+
+def test_graphed_helper_training_step_padded_stack():
+    """Forward and backward of a padded bidirectional stack (the 4-layer d=512 L=128 B=32
+    configuration at half its depth and batch) recorded with sru_amd.graphed in training mode:
+    outputs and every parameter gradient of three replays on fresh inputs against eager runs."""
+    import sru_amd
+    torch.manual_seed(8)
+    L, B = 128, 16
+    model = sru_amd.SRU(512, 512, num_layers=2, bidirectional=True).cuda().train()
+    mk_mask = lambda: torch.arange(L, device="cuda")[:, None] >= torch.randint(32, L + 1, (B,), device="cuda")[None, :]
+    x0, m0 = torch.randn(L, B, 512, device="cuda"), mk_mask()
+    fast = sru_amd.graphed(model, x0, mask_pad=m0)
+    assert fast.training
+    for replay in range(3):
+        x, m = torch.randn(L, B, 512, device="cuda"), mk_mask()
+        probe = torch.randn(L, B, 1024, device="cuda")
+        model.zero_grad(set_to_none=True)
+        h, c = model(x, mask_pad=m)
+        ((h * probe).sum() + c.sum()).backward()
+        eager = [h.detach().clone(), c.detach().clone()] + [p.grad.clone() for p in model.parameters()]
+        model.zero_grad(set_to_none=True)
+        torch.cuda.synchronize()
+        h, c = fast(x, mask_pad=m)
+        ((h * probe).sum() + c.sum()).backward()
+        torch.cuda.synchronize()
+        got = [h.detach(), c.detach()] + [p.grad for p in model.parameters()]
+        for a, b in zip(got, eager):
+            assert float((a - b).abs().max()) <= 1e-6 * max(1.0, float(b.abs().max())), replay
