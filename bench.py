@@ -307,6 +307,9 @@ def main():
                     help="with a stack workload: use torch.nn.LayerNorm's kernels instead of this package's")
     ap.add_argument("--shape", default=None, metavar="L,B,d,dirs",
                     help="side measurement at another shape (k=3 forward + backward, no padding); replaces --workload")
+    ap.add_argument("--fixed-length", type=int, default=0,
+                    help="side measurement with a padded workload: every sequence has this length (default: "
+                         "lengths uniform in [L/4, L])")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also time a plain device copy of 1 GiB (context for the roofline figures "
@@ -378,6 +381,8 @@ def main():
     pad = None
     if padded:
         lens = torch.randint(L // 4, L + 1, (B,), device=dev, generator=g)
+        if args.fixed_length:
+            lens = torch.full((B,), args.fixed_length, device=dev)
         pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :]).view(torch.uint8).contiguous()
     gwc = torch.empty(L, B, 2 * Dp, device=dev, dtype=tdt) if custom else torch.empty(2 * Dp, device=dev)
     gb = torch.empty(2 * Dp, device=dev)

@@ -36,7 +36,10 @@ constexpr int64_t kPairBelow = SRU_AMD_PAIR_BELOW;
 // Lane-pair kernels (sru_split.h): 16-bit streams, d a multiple of 32, at most 1024 wavefronts of 32
 // columns, every stream 16-byte aligned, state kept as checkpoints or not at all.
 constexpr int kSplitNbuf = 2;   // chunks (of 16 steps) in flight per wavefront
-inline bool split_wanted(int64_t ncols, int32_t d) { return d % kSplitCols == 0 && ncols / kSplitCols <= 1024; }
+#ifndef SRU_AMD_SPLIT_MAX_WAVES   // (set by tuning builds only)
+#define SRU_AMD_SPLIT_MAX_WAVES 1024
+#endif
+inline bool split_wanted(int64_t ncols, int32_t d) { return d % kSplitCols == 0 && ncols / kSplitCols <= SRU_AMD_SPLIT_MAX_WAVES; }
 
 inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -352,6 +352,25 @@ struct BwdParams {
     int32_t act, custom;
 };
 
+// Every field of the parameter block is read at the top of a kernel. Left alone, the compiler
+// fetches each field from the kernel-argument segment right before its first use, which makes the
+// prologue a chain of dependent scalar-memory round trips (one per basic block that needs a new
+// field); pinned here, the fields arrive with a few wide scalar loads behind one wait.
+#define SRU_AMD_PIN(v) asm volatile("" ::"s"(v))
+__device__ __forceinline__ void fetch_params_early(const FwdParams &p) {
+    SRU_AMD_PIN(p.u); SRU_AMD_PIN(p.x); SRU_AMD_PIN(p.wc); SRU_AMD_PIN(p.bias); SRU_AMD_PIN(p.c0);
+    SRU_AMD_PIN(p.mask_c); SRU_AMD_PIN(p.pad); SRU_AMD_PIN(p.scale_x); SRU_AMD_PIN(p.h); SRU_AMD_PIN(p.c);
+    SRU_AMD_PIN(p.c_last); SRU_AMD_PIN(p.ckpt); SRU_AMD_PIN(p.L); SRU_AMD_PIN(p.B); SRU_AMD_PIN(p.ncols);
+    SRU_AMD_PIN(p.d); SRU_AMD_PIN(p.Dp);
+}
+__device__ __forceinline__ void fetch_params_early(const BwdParams &p) {
+    SRU_AMD_PIN(p.u); SRU_AMD_PIN(p.x); SRU_AMD_PIN(p.wc); SRU_AMD_PIN(p.bias); SRU_AMD_PIN(p.c0);
+    SRU_AMD_PIN(p.mask_c); SRU_AMD_PIN(p.pad); SRU_AMD_PIN(p.scale_x); SRU_AMD_PIN(p.c); SRU_AMD_PIN(p.gh);
+    SRU_AMD_PIN(p.ckpt); SRU_AMD_PIN(p.glast); SRU_AMD_PIN(p.gu); SRU_AMD_PIN(p.gx); SRU_AMD_PIN(p.gwc_steps);
+    SRU_AMD_PIN(p.ginit); SRU_AMD_PIN(p.partial); SRU_AMD_PIN(p.L); SRU_AMD_PIN(p.B); SRU_AMD_PIN(p.ncols);
+    SRU_AMD_PIN(p.d); SRU_AMD_PIN(p.Dp);
+}
+
 // The loop body must stay one straight line of code for the compiler to keep the ring
 // in fixed registers and count outstanding loads (a uniform branch inside it makes the
 // inserted waits drain the ring at every step). The fast kernels therefore take "is
@@ -571,6 +590,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
     // issue slots, and reading a flag back from its lane costs one instruction more per step.
     constexpr bool PAD_BY_LANE = HAS_PAD && UNI && !PAIR;
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
+    fetch_params_early(p);
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
     using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c: two elements per column
@@ -644,7 +664,11 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
 #pragma unroll
         for (int i = 0; i < TC; ++i) {
             if (i < n) {
-                const bool padded = (PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i]) != 0;
+                // a padded step keeps the state and emits zero, through bit masks: with selects on a flag
+                // that is uniform over the wavefront the compiler branches around the arithmetic, which
+                // cuts the chunk into one basic block per step and column and serialises the columns
+                const uint32_t flag = PAD_BY_LANE ? (uint32_t)__builtin_amdgcn_readlane((int)k.pad[0], i) : k.pad[i];
+                const uint32_t keep = 0u - (uint32_t)(flag != 0);   // all ones at a padded step
                 float hv[COLS], cv[COLS], uu[COLS * K], xx[COLS] = {};
                 SU::unpack(k.u[i], q, uu);
                 if (SKIP == 1) S1::unpack(k.x[i], q, xx);
@@ -664,8 +688,8 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
                     } else {
                         out = val * m[c] * g2;
                     }
-                    cur[c] = padded ? cur[c] : cn;
-                    hv[c] = padded ? 0.0f : out;
+                    cur[c] = __builtin_bit_cast(float, (__builtin_bit_cast(uint32_t, cur[c]) & keep) | (__builtin_bit_cast(uint32_t, cn) & ~keep));
+                    hv[c] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, out) & ~keep);
                     cv[c] = cur[c];
                 }
                 const int64_t e = ef + (s0 + i) * es;
@@ -946,6 +970,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
     using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
     using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c and its gradient: two elements per column
+    fetch_params_early(p);
     // the wavefront's index in the launch (scalar), and the lane's in the wavefront
     const uint32_t wg = blockIdx.x * (blockDim.x / kBlock) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kBlock));
     const uint32_t wlane = threadIdx.x % kBlock;
@@ -1017,13 +1042,25 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
         // compiler keep the initial state in scratch memory and select between addresses itself)
         // (without an initial state the first chunk starts from zero; its load reads checkpoint row 0,
         // which always exists, and drops the value)
-        const bool zero_start = ch == 0 && !p.c0;
-        const float *from = (ch == 0 && p.c0) ? p.c0 + col : p.ckpt + (ch > 0 ? ch - 1 : 0) * p.ncols + col;
-#pragma unroll
-        for (int c = 0; c < COLS; ++c) {
-            const float v = from[c];
-            k.cstart[c] = zero_start ? 0.0f : v;
+        // (the value is dropped with a bit mask: a select makes the compiler branch around the load,
+        // inside the pipelined loop)
+        const uint32_t keep = (ch == 0 && !p.c0) ? 0u : ~0u;
+        // The address is one of two bases. As a select it becomes a scalar branch that cuts the loop
+        // body in two, which the one-column-per-lane kernels like (measured 8 % faster at 512
+        // wavefronts, level at 2 048) and the two-columns-per-lane kernels do not (6 % slower at
+        // 1 024 wavefronts): those blend the bases with bit masks instead.
+        const float *from;
+        if constexpr (COLS == 2) {
+            const uintptr_t use_c0 = (ch == 0 && p.c0) ? ~(uintptr_t)0 : (uintptr_t)0;
+            const uintptr_t base = (reinterpret_cast<uintptr_t>(p.c0) & use_c0) |
+                                   (reinterpret_cast<uintptr_t>(p.ckpt + (ch > 0 ? ch - 1 : 0) * p.ncols) & ~use_c0);
+            from = reinterpret_cast<const float *>(base) + col;
+        } else {
+            from = (ch == 0 && p.c0) ? p.c0 + col : p.ckpt + (ch > 0 ? ch - 1 : 0) * p.ncols + col;
         }
+#pragma unroll
+        for (int c = 0; c < COLS; ++c)
+            k.cstart[c] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, from[c]) & keep);
     };
 
     auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
