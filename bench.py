@@ -211,8 +211,9 @@ def run_stack(args):
 def run_layer_norm(args):
     """Side measurement: the layer-norm kernels next to the recurrence, through the C ABI, at the
     row count and width of the headline layer (16 384 rows of 2 048 features). Forward and backward
-    (the backward call includes the two launches that add the workgroups' weight / bias sums) are
-    timed with HIP events on rotating buffer sets; the roofline is HBM, bytes = rows read + written."""
+    (the backward call includes the launch that adds the workgroups' weight / bias sums) are
+    timed with HIP events on rotating buffer sets; the roofline is HBM, bytes = rows read + written,
+    plus, for the backward call, the workgroups' partial sums written once and read once."""
     import torch
     from sru_amd import _lib
     rows, D = 256 * 64, 2048
@@ -264,14 +265,14 @@ def run_layer_norm(args):
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     f_us = sum(a.elapsed_time(m) for a, m, _ in marks[args.warmup:]) * 1e3 / args.steps
     b_us = sum(m.elapsed_time(e) for _, m, e in marks[args.warmup:]) * 1e3 / args.steps
-    f_bytes, b_bytes = 2 * es * rows * D, 3 * es * rows * D
+    f_bytes, b_bytes = 2 * es * rows * D, 3 * es * rows * D + 2 * nbytes
     gbs = lambda nb, us: nb / (us * 1e-6) / 1e9
     print(json.dumps({
         "metric": "layer norm rows/s (side measurement)", "value": rows / (ms_step * 1e-3), "unit": "rows/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": f"layer norm forward + backward, {rows} rows of {D} features, {args.dtype} in and out"},
-        "roofline": {"bound": "hbm", "kernel": "layer_norm_backward (+ reduce_rows x 2)", "achieved": gbs(b_bytes, b_us),
+        "roofline": {"bound": "hbm", "kernel": "layer_norm_backward (+ reduce_rows)", "achieved": gbs(b_bytes, b_us),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs(b_bytes, b_us) / HBM_PEAK_GBS, "traffic": None,
                      "avg_us": b_us},
         "kernels": {"layer_norm_forward": {"avg_us": f_us, "algorithmic_GBps": gbs(f_bytes, f_us),
@@ -477,6 +478,11 @@ def main():
     ms_step = (t1 - t0) * 1e3 / args.steps
     fwd_us = 1e3 * sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     bwd_us = 1e3 * sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    # spread of the timed region: per-step times between the events that open consecutive steps
+    # (the last step: from its own first to its last event)
+    per_step = [ev[i][0].elapsed_time(ev[i + 1][0]) for i in range(args.steps - 1)] + [ev[-1][0].elapsed_time(ev[-1][2])]
+    spread = {"min": min(per_step), "median": float(np.median(per_step)), "max": max(per_step),
+              "source": "HIP events on the launch stream, one value per timed step"}
     # HBM bytes per backward launch as the hardware counters saw them: NOT measured by this run
     # (counters need a rocprofv3 --pmc session) but replayed from the committed summary of such
     # sessions on this same command; the file is named in the output
@@ -522,6 +528,7 @@ def main():
         "value": L * B / (ms_step * 1e-3),
         "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
+        "ms_per_step_spread": spread,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic",
         "config": {"workload": name, "length": L, "batch": B, "hidden_per_direction": d,

@@ -23,7 +23,7 @@
  *
  * Layouts (those of the reference)
  *   U        (L, B, D', k)      k innermost; D' = dirs * hidden
- *   x, h, c, grad_h, grad_x     (L, B, D')
+ *   x, h, c, grad_h, grad_x     (L, B, D')            (x, grad_x: see shape->x_dtype)
  *   weight_c (2, D') float, or, when is_custom, (L, B, D', 2) in `dtype`
  *   bias     (2, D') float
  *   c_init, mask_c, c_last, grad_last, grad_init   (B, D') float
@@ -100,7 +100,18 @@ typedef struct sru_amd_shape {
                               *   kernels of every shape are built for; with 0 / 1 the 16-bit
                               *   kernels for few columns and the checkpoint backward kernels are
                               *   not available. No counterpart in the reference. */
+    int32_t x_dtype;         /* element type of x and grad_x: SRU_AMD_X_AS_STREAMS (0): `dtype`, like
+                              * every other stream; SRU_AMD_X_F32: float, next to 16-bit streams -
+                              * under autocast the reference hands the recurrence a float32 x beside
+                              * the 16-bit U (sru/ops.py:116-127 casts both to float32; here neither
+                              * is cast). Needs skip_type 1 (otherwise x is not read and the field is
+                              * ignored), is_custom 0, activation_type 0, an even `hidden`, and the
+                              * state as checkpoints or not at all (BAD_FLAGS otherwise). With dtype
+                              * SRU_AMD_F32 both values mean the same. */
 } sru_amd_shape;
+
+#define SRU_AMD_X_AS_STREAMS 0
+#define SRU_AMD_X_F32 1
 
 #define SRU_AMD_STATE_INTERVAL 8
 

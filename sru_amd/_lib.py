@@ -15,6 +15,7 @@ STATIC_MAX_COLUMNS = 262144   # SRU_AMD_STATIC_MAX_COLUMNS
 NORM_MAX_FEATURES = 4096       # SRU_AMD_NORM_MAX_FEATURES
 
 F32, F16, BF16 = 0, 1, 2
+X_AS_STREAMS, X_F32 = 0, 1   # SRU_AMD_X_AS_STREAMS, SRU_AMD_X_F32
 
 
 class Shape(ctypes.Structure):
@@ -30,6 +31,7 @@ class Shape(ctypes.Structure):
         ("is_custom", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
         ("state_interval", ctypes.c_int32),
+        ("x_dtype", ctypes.c_int32),
     ]
 
 

@@ -44,6 +44,11 @@ size_t elem_size(int dtype) { return dtype == SRU_AMD_F32 ? 4 : 2; }
 
 bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// x (and grad_x) is float while the other streams are 16-bit
+bool x_is_float_beside_16bit(const sru_amd_shape &s) {
+    return s.dtype != SRU_AMD_F32 && s.x_dtype == SRU_AMD_X_F32 && s.skip_type == 1;
+}
+
 // Shape and flag rules; those on k / skip_type are the device-side asserts of the
 // reference's general kernels (sru/csrc/sru_cuda_kernel.cu:397-399).
 int check_shape(const sru_amd_shape *s) {
@@ -68,6 +73,11 @@ int check_shape(const sru_amd_shape *s) {
         if (s->is_custom != 0 && s->activation_type != 0) return SRU_AMD_ERR_BAD_FLAGS;
         if (s->dtype != SRU_AMD_F32 && s->hidden % 2 != 0) return SRU_AMD_ERR_BAD_FLAGS;
     }
+    if (s->x_dtype != SRU_AMD_X_AS_STREAMS && s->x_dtype != SRU_AMD_X_F32) return SRU_AMD_ERR_BAD_DTYPE;
+    // a float x next to 16-bit streams exists in the chunked kernels for the plain layer only
+    // (and for the state as checkpoints or not at all, which the entry points check)
+    if (x_is_float_beside_16bit(*s) && (s->is_custom != 0 || s->activation_type != 0 || s->hidden % 2 != 0))
+        return SRU_AMD_ERR_BAD_FLAGS;
     // D' must fit an int, the grid must fit 2^31-1 workgroups and the largest stream
     // (L*B*D'*k elements) must stay far inside the 64-bit byte offsets the kernels use.
     const int64_t lim = INT64_C(1) << 31;
@@ -94,8 +104,11 @@ int backward_core(const sru_amd_shape *shape, const void *u, const void *x, cons
     const size_t es = elem_size(s.dtype);
     const size_t group = (s.k == 4) ? 4 * es : es;
     const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
+    const bool x_float = x_is_float_beside_16bit(s);
+    if (x_float && !ckpt) return SRU_AMD_ERR_BAD_FLAGS;
+    const size_t xs = x_float ? 4 : es;
     if (!aligned(u, group) || !aligned(grad_u, group) || !aligned(c, ckpt ? 4 : es) || !aligned(grad_h, es) ||
-        (s.skip_type == 1 && (!aligned(x, es) || !aligned(grad_x, es))) ||
+        (s.skip_type == 1 && (!aligned(x, xs) || !aligned(grad_x, xs))) ||
         !aligned(weight_c, s.is_custom ? 2 * es : 4) || !aligned(grad_wc, s.is_custom ? 2 * es : 4) ||
         !aligned(bias, 4) || (c_init && !aligned(c_init, 4)) || (grad_last && !aligned(grad_last, 4)) || !aligned(grad_bias, 4) ||
         !aligned(grad_init, 4) || (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
@@ -115,7 +128,7 @@ int backward_core(const sru_amd_shape *shape, const void *u, const void *x, cons
     p.gu = grad_u; p.gx = grad_x; p.gwc_steps = s.is_custom ? grad_wc : nullptr;
     p.ginit = grad_init; p.partial = partial;
     p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
-    p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
+    p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom; p.x_float = x_float;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const hipError_t err = s.dtype == SRU_AMD_F32   ? launch_backward<float>(s, p, st)
@@ -160,8 +173,12 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
     const size_t es = elem_size(s.dtype);
     const size_t group = (s.k == 4) ? 4 * es : es;  // a k=4 group moves as one vector
     const bool ckpt = s.state_interval == SRU_AMD_STATE_INTERVAL;
+    const bool x_float = x_is_float_beside_16bit(s);
+    if (x_float && c && !ckpt) return SRU_AMD_ERR_BAD_FLAGS;
+    // (a float x still travels with 16-bit streams that move two columns at a time)
+    if (x_float && (!aligned(u, s.k == 4 ? 16 : 4) || !aligned(h, 4))) return SRU_AMD_ERR_MISALIGNED;
     if (!aligned(u, group) || !aligned(h, es) || (c && !aligned(c, ckpt ? 4 : es)) ||
-        (s.skip_type == 1 && !aligned(x, es)) || !aligned(weight_c, s.is_custom ? 2 * es : 4) ||
+        (s.skip_type == 1 && !aligned(x, x_float ? 4 : es)) || !aligned(weight_c, s.is_custom ? 2 * es : 4) ||
         !aligned(bias, 4) || (c_init && !aligned(c_init, 4)) || !aligned(c_last, 4) ||
         (mask_c && !aligned(mask_c, 4)) || (scale_x && !aligned(scale_x, 4)))
         return SRU_AMD_ERR_MISALIGNED;
@@ -178,7 +195,7 @@ int sru_amd_forward(const sru_amd_shape *shape, const void *u, const void *x, co
     p.c = ckpt ? nullptr : c;
     p.ckpt = ckpt ? static_cast<float *>(c) : nullptr;
     p.L = s.length; p.B = s.batch; p.d = (int32_t)s.hidden; p.Dp = (int32_t)(s.hidden * s.dirs);
-    p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom;
+    p.ncols = s.batch * p.Dp; p.act = s.activation_type; p.custom = s.is_custom; p.x_float = x_float;
 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const hipError_t err = s.dtype == SRU_AMD_F32   ? launch_forward<float>(s, p, st)

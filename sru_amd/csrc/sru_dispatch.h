@@ -89,47 +89,51 @@ inline bool wave_uniform(int32_t d, int cols) { return d % (kBlock * cols) == 0;
 
 // X: the template bits fixed so far (pairing, then uniformity, then activation); the run-time
 // properties are turned into template bits one at a time.
-template <typename T, int K, int SKIP, int COLS, int X = 0, int STAGE = 0>
+// TX: element type of x / grad_x (T, or float next to 16-bit streams: those builds exist for the
+// identity activation, checkpointed or no state, no per-step weight_c; callers start them at STAGE 1).
+template <typename T, int K, int SKIP, int COLS, int X = 0, int STAGE = 0, typename TX = T>
 hipError_t fast_forward(const FwdParams &p, hipStream_t st) {
     if constexpr (STAGE == 0 && (X & kCustom) != 0) {   // (a per-step weight_c with tanh runs the general kernels)
-        return fast_forward<T, K, SKIP, COLS, X, 1>(p, st);
+        return fast_forward<T, K, SKIP, COLS, X, 1, TX>(p, st);
     } else if constexpr (STAGE == 0) {
-        return p.act ? fast_forward<T, K, SKIP, COLS, X | kTanh, 1>(p, st) : fast_forward<T, K, SKIP, COLS, X, 1>(p, st);
+        return p.act ? fast_forward<T, K, SKIP, COLS, X | kTanh, 1, TX>(p, st) : fast_forward<T, K, SKIP, COLS, X, 1, TX>(p, st);
     } else if constexpr (STAGE == 1) {
-        return wave_uniform(p.d, COLS) ? fast_forward<T, K, SKIP, COLS, X | kUniform, 2>(p, st)
-                                       : fast_forward<T, K, SKIP, COLS, X, 2>(p, st);
+        return wave_uniform(p.d, COLS) ? fast_forward<T, K, SKIP, COLS, X | kUniform, 2, TX>(p, st)
+                                       : fast_forward<T, K, SKIP, COLS, X, 2, TX>(p, st);
     } else if constexpr (STAGE == 2) {
-        return p.pad ? fast_forward<T, K, SKIP, COLS, X | kHasPad, 3>(p, st) : fast_forward<T, K, SKIP, COLS, X, 3>(p, st);
+        return p.pad ? fast_forward<T, K, SKIP, COLS, X | kHasPad, 3, TX>(p, st) : fast_forward<T, K, SKIP, COLS, X, 3, TX>(p, st);
     } else {
         constexpr int TC = kCkptInterval;
         const int most = max_waves_per_group<T>(X);
         // what is kept for the backward pass: checkpoints, the state after every step, or nothing
-        if (p.ckpt) return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt | kCkpt, COLS, TC>, p.ncols, COLS, most, st, p);
-        if constexpr ((X & kCustom) == 0) {   // (with a per-step weight_c the state after every step is the general kernels')
+        if (p.ckpt) return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt | kCkpt, COLS, TC, TX>, p.ncols, COLS, most, st, p);
+        // (with a per-step weight_c the state after every step is the general kernels'; with a float x
+        // next to 16-bit streams it is refused before)
+        if constexpr ((X & kCustom) == 0 && sizeof(TX) == sizeof(T)) {
             if (p.c) return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt | kKeepC, COLS, TC>, p.ncols, COLS, most, st, p);
         }
-        return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt, COLS, TC>, p.ncols, COLS, most, st, p);
+        return launch_grouped(forward_scan_chunked<T, K, SKIP, X | kNt, COLS, TC, TX>, p.ncols, COLS, most, st, p);
     }
 }
 
-template <typename T, int K, int SKIP, int COLS, int X = 0, int STAGE = 0>
+template <typename T, int K, int SKIP, int COLS, int X = 0, int STAGE = 0, typename TX = T>
 hipError_t fast_backward(const BwdParams &p, hipStream_t st) {
     if constexpr (STAGE == 0 && (X & kCustom) != 0) {
-        return fast_backward<T, K, SKIP, COLS, X, 1>(p, st);
+        return fast_backward<T, K, SKIP, COLS, X, 1, TX>(p, st);
     } else if constexpr (STAGE == 0) {
-        return p.act ? fast_backward<T, K, SKIP, COLS, X | kTanh, 1>(p, st) : fast_backward<T, K, SKIP, COLS, X, 1>(p, st);
+        return p.act ? fast_backward<T, K, SKIP, COLS, X | kTanh, 1, TX>(p, st) : fast_backward<T, K, SKIP, COLS, X, 1, TX>(p, st);
     } else if constexpr (STAGE == 1) {
-        return p.pad ? fast_backward<T, K, SKIP, COLS, X | kHasPad, 2>(p, st) : fast_backward<T, K, SKIP, COLS, X, 2>(p, st);
+        return p.pad ? fast_backward<T, K, SKIP, COLS, X | kHasPad, 2, TX>(p, st) : fast_backward<T, K, SKIP, COLS, X, 2, TX>(p, st);
     } else {
-        if constexpr ((X & (kPair | kCustom)) == 0) {   // (lane pairing and the weight_c stream exist in the chunked kernels only)
+        if constexpr ((X & (kPair | kCustom)) == 0 && sizeof(TX) == sizeof(T)) {   // (lane pairing, the weight_c stream and a float x exist in the chunked kernels only)
             // reference-style state: the ring kernel reads it step by step
             if (!p.ckpt) return launch_grouped(backward_scan<T, K, SKIP, X | kNt, COLS, kRingDepth>, p.ncols, COLS, 4, st, p);
         }
         constexpr int TC = kCkptInterval;
         const int most = max_waves_per_group<T>(X);
         if (wave_uniform(p.d, COLS))
-            return launch_grouped(backward_scan_ckpt<T, K, SKIP, X | kNt | kUniform, COLS, TC>, p.ncols, COLS, most, st, p);
-        return launch_grouped(backward_scan_ckpt<T, K, SKIP, X | kNt, COLS, TC>, p.ncols, COLS, most, st, p);
+            return launch_grouped(backward_scan_ckpt<T, K, SKIP, X | kNt | kUniform, COLS, TC, TX>, p.ncols, COLS, most, st, p);
+        return launch_grouped(backward_scan_ckpt<T, K, SKIP, X | kNt, COLS, TC, TX>, p.ncols, COLS, most, st, p);
     }
 }
 
@@ -176,6 +180,13 @@ hipError_t general_backward(const BwdParams &p, hipStream_t st) {
 template <typename T, int K, int SKIP>
 hipError_t pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
+        if constexpr (SKIP == 1) {
+            if (p.x_float) {   // a float x next to 16-bit streams: chunked kernels only (the flag combinations were checked before)
+                if (p.act || p.c || !pair_ok<T, K>(s, {p.u}, {p.h}) || !aligned_to(p.x, 4)) return hipErrorInvalidValue;
+                if (p.ncols / 2 < kPairBelow) return fast_forward<T, K, SKIP, 1, kPair, 1, float>(p, st);
+                return fast_forward<T, K, SKIP, 2, 0, 1, float>(p, st);
+            }
+        }
         if (!p.c && split_wanted(p.ncols, p.d) && all_aligned_16({p.u, p.x, p.h}))
             return split_forward<T, K, SKIP>(p, st);
         if (!pair_ok<T, K>(s, {p.u}, {p.x, p.h, p.c}))
@@ -190,6 +201,14 @@ hipError_t pick_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t 
 template <typename T, int K, int SKIP>
 hipError_t pick_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
+        if constexpr (SKIP == 1) {
+            if (p.x_float) {
+                if (p.act || !p.ckpt || !pair_ok<T, K>(s, {p.u, p.gu}, {p.gh}) || !aligned_to(p.x, 4) || !aligned_to(p.gx, 4))
+                    return hipErrorInvalidValue;
+                if (p.ncols / 2 < kPairBelow) return fast_backward<T, K, SKIP, 1, kPair, 1, float>(p, st);
+                return fast_backward<T, K, SKIP, 2, 0, 1, float>(p, st);
+            }
+        }
         if (p.ckpt && split_wanted(p.ncols, p.d) && all_aligned_16({p.u, p.x, p.gh, p.gu, p.gx}))
             return split_backward<T, K, SKIP>(p, st);
         if (!pair_ok<T, K>(s, {p.u, p.gu}, {p.x, p.c, p.gh, p.gx}))   // p.c is null with checkpoints

@@ -10,9 +10,12 @@
 // 16-byte vectors per lane, 16-bit rows as one; workgroups walk rows with a stride of the grid and
 // load the next row while they reduce the current one. Statistics are float: mean first, then the
 // variance of the centred values (wavefront reductions combined through LDS in wavefront order).
-// The backward kernel keeps each lane's share of the weight / bias gradient sums in registers over
-// the rows its workgroup visits and leaves one partial row per workgroup; reduce_rows() then adds
-// the workgroups in index order, in double: bit-reproducible.
+// The backward kernel runs at most one workgroup per compute unit: 16 wavefronts that form several
+// row groups, each working like a workgroup of the forward kernel on rows of its own. Every lane
+// keeps its share of the weight / bias gradient sums in registers over the rows its group visits;
+// at the end the groups add their shares through LDS in group order and the workgroup leaves one
+// partial row (at most 256 in all, 4 MB at 2 048 features); reduce_rows() then adds the workgroups
+// in index order, in double, in one launch: bit-reproducible.
 #include "sru_amd.h"
 
 #include <hip/hip_runtime.h>
@@ -107,8 +110,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 // Rows a workgroup handles per trip: their loads are in flight together and their sums share a barrier.
 constexpr int kRowsPer = 2;
 
-// Sums over the workgroup (the WAVES wavefronts that share a row) of N values at once, the
-// wavefronts' shares added in wavefront order. `red` holds N * WAVES floats and must not be
+// Sums over the WAVES wavefronts that share a row (a whole workgroup, or one row group of it; the
+// barrier is the workgroup's) of N values at once, the wavefronts' shares added in wavefront order. `red` holds N * WAVES floats and must not be
 // rewritten before every thread has read it (the callers alternate two arrays so that the next
 // barrier provides that).
 template <int WAVES, int N>
@@ -118,7 +121,7 @@ __device__ __forceinline__ void block_sums(float (&v)[N], float *red) {
     if constexpr (WAVES > 1) {
         if ((threadIdx.x & (kLanes - 1)) == 0) {
 #pragma unroll
-            for (int n = 0; n < N; ++n) red[n * WAVES + (threadIdx.x >> 6)] = v[n];
+            for (int n = 0; n < N; ++n) red[n * WAVES + ((threadIdx.x >> 6) % WAVES)] = v[n];
         }
         __syncthreads();
 #pragma unroll
@@ -203,15 +206,20 @@ layer_norm_forward(const TI *x, const float *gamma, const float *beta, TO *y, fl
 }
 
 // dx = rstd * (g - mean(g) - xhat * mean(g * xhat)) with g = dy * gamma, xhat = (x - mean) * rstd;
-// partial[block] = (sum over the block's rows of dy * xhat, sum of dy), each D floats: every feature
-// belongs to one lane of the workgroup, which adds its rows in the order it visits them.
-template <typename TI, typename TG, typename TD, int WAVES>
-__global__ void __launch_bounds__(kLanes * WAVES)
+// partial[block] = (sum over the block's rows of dy * xhat, sum of dy), each D floats.
+// A workgroup is GROUPS row groups of WAVES wavefronts; a group owns kRowsPer consecutive rows per
+// trip, every lane 8 consecutive features of each, and the groups of all workgroups walk the rows
+// with a stride of the launch. Every feature belongs to one lane of each group, which adds its rows
+// in the order it visits them; the groups' sums are added in group order at the end.
+template <typename TI, typename TG, typename TD, int WAVES, int GROUPS>
+__global__ void __launch_bounds__(kLanes * WAVES * GROUPS)
 layer_norm_backward(const TI *x, const float *gamma, const float *mean, const float *rstd, const TG *dy, TD *dx,
                     float *partial, int64_t rows, int32_t D) {
     constexpr int R = kRowsPer;
-    __shared__ float red[2][2 * R * WAVES];   // alternate by trip: one barrier per trip
-    const int e = threadIdx.x * kPer;
+    __shared__ float red[2][GROUPS][2 * R * WAVES];   // alternate by trip: one barrier per trip
+    __shared__ float acc[2 * kPass * WAVES];            // the groups' weight / bias sums, added in group order
+    const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / (kLanes * WAVES)));
+    const int e = (int)(threadIdx.x % (kLanes * WAVES)) * kPer;
     const bool active = e < D;
     float g[kPer] = {}, dg[kPer] = {}, db[kPer] = {};
     if (active) load8<float>(gamma + e, g);
@@ -220,24 +228,30 @@ layer_norm_backward(const TI *x, const float *gamma, const float *mean, const fl
     const TI *my_x = x + ec;
     const TG *my_dy = dy + ec;
     const int64_t last = rows - 1;
+    const int64_t stride = (int64_t)gridDim.x * GROUPS * R;
     Raw<TI> nx[R];
     Raw<TG> nd[R];
-    int64_t row = (int64_t)blockIdx.x * R;
+    // `first` is the first row of the workgroup's trip (the same for all its groups, so that every
+    // wavefront makes the same number of trips and meets the others at the barriers); a group past
+    // the last row repeats the last row and drops it
+    int64_t first = (int64_t)blockIdx.x * GROUPS * R;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int64_t at = (row + r < last ? row + r : last) * D;
+        const int64_t row = first + grp * R + r;
+        const int64_t at = (row < last ? row : last) * D;
         nx[r].load(my_x + at);
         nd[r].load(my_dy + at);
     }
     int parity = 0;
-    for (; row < rows; row += (int64_t)gridDim.x * R, parity ^= 1) {
+    for (; first < rows; first += stride, parity ^= 1) {
+        const int64_t row = first + grp * R;
         float xh[R][kPer], gy[R][kPer], sums[2 * R], rs[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             nx[r].unpack(xh[r]);
             nd[r].unpack(gy[r]);
         }
-        const int64_t after = row + (int64_t)gridDim.x * R;
+        const int64_t after = row + stride;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const int64_t at = (after + r < last ? after + r : last) * D;
@@ -265,7 +279,7 @@ layer_norm_backward(const TI *x, const float *gamma, const float *mean, const fl
             sums[2 * r] = s1;
             sums[2 * r + 1] = s2;
         }
-        block_sums<WAVES, 2 * R>(sums, red[parity]);
+        block_sums<WAVES, 2 * R>(sums, red[parity][grp]);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (row + r >= rows || !active) continue;
@@ -276,44 +290,87 @@ layer_norm_backward(const TI *x, const float *gamma, const float *mean, const fl
             store8<TD>(dx + (row + r) * D + e, o);
         }
     }
-    if (active) {
+    // the groups' shares, added in group order
+#pragma unroll
+    for (int gi = 0; gi < GROUPS; ++gi) {
+        if (grp == gi && active) {
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                acc[e + i] = (gi == 0 ? 0.f : acc[e + i]) + dg[i];
+                acc[kPass * WAVES + e + i] = (gi == 0 ? 0.f : acc[kPass * WAVES + e + i]) + db[i];
+            }
+        }
+        __syncthreads();
+    }
+    if (grp == 0 && active) {
         float *out = partial + (int64_t)blockIdx.x * 2 * D;
+#pragma unroll
+        for (int i = 0; i < kPer; ++i) {
+            dg[i] = acc[e + i];
+            db[i] = acc[kPass * WAVES + e + i];
+        }
         store8<float>(out + e, dg);
         store8<float>(out + D + e, db);
     }
 }
 
-// out[slab][e] = sum over the slab's rows r of partial[r][e]; slab = blockIdx.y takes rows
-// [slab * chunk, (slab + 1) * chunk). One workgroup per 64 columns and slab; its 16 wavefronts take
-// every 16th row each, accumulate in double and are combined through LDS in a fixed order. Many
-// rows go in two launches (float rows -> kSlabs double rows -> one float row), few in one.
+// out[e] = sum over the rows r of partial[r][e]. One workgroup per 64 columns; its 16 wavefronts
+// take every 16th row each, accumulate in double and are combined through LDS in a fixed order.
 constexpr int kRowSlices = 16;
-constexpr int kSlabs = 16;
-template <typename TIN, typename TOUT>
 __global__ void __launch_bounds__(kLanes * kRowSlices)
-reduce_rows(const TIN *partial, TOUT *out, int32_t nrows, int32_t width, int32_t chunk) {
+reduce_rows(const float *partial, float *out, int32_t nrows, int32_t width) {
     __shared__ double part[kRowSlices][kLanes];
     const int lane = threadIdx.x & (kLanes - 1), slice = threadIdx.x >> 6;
     const int e = blockIdx.x * kLanes + lane;
-    const int first = blockIdx.y * chunk;
-    const int end = first + chunk < nrows ? first + chunk : nrows;
     double s = 0.0;
-    if (e < width)
-        for (int r = first + slice; r < end; r += kRowSlices) s += (double)partial[(int64_t)r * width + e];
+    if (e < width) {
+        // the loads of a batch are issued together (addresses clamped, surplus values dropped), then added in row order
+        constexpr int kBatch = 8;
+        for (int r0 = slice; r0 < nrows; r0 += kRowSlices * kBatch) {
+            float v[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int r = r0 + i * kRowSlices;
+                v[i] = partial[(int64_t)(r < nrows ? r : nrows - 1) * width + e];
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) s += (r0 + i * kRowSlices < nrows) ? (double)v[i] : 0.0;
+        }
+    }
     part[slice][lane] = s;
     __syncthreads();
     if (slice == 0 && e < width) {
         double total = part[0][lane];
 #pragma unroll
         for (int i = 1; i < kRowSlices; ++i) total += part[i][lane];
-        out[(int64_t)blockIdx.y * width + e] = (TOUT)total;
+        out[e] = (float)total;
     }
 }
 
-// Workgroups of a launch: each walks groups of kRowsPer rows with a stride of the grid.
+// wavefronts per row: 8 features per lane
+inline int norm_waves(int32_t D) {
+    const int need = (D + kPass - 1) / kPass;
+    return need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
+}
+
+// Workgroups of a forward launch: each walks groups of kRowsPer rows with a stride of the grid.
 int norm_blocks(int64_t rows) {
     const int64_t groups = (rows + kRowsPer - 1) / kRowsPer;
     return (int)(groups < 1024 ? groups : 1024);
+}
+
+// The backward kernel: 16 wavefronts per workgroup (16 / waves-per-row row groups) and at most one
+// workgroup per compute unit for 16-bit rows, 8 wavefronts and at most two workgroups for float rows
+// (measured at 16 384 x 2 048: bf16 44 us against 48 us with 8, float 84 us against 89 us with 16),
+// so that the partial rows stay few; rows of more than 2 048 features (8 wavefronts per row) form
+// one group per workgroup of 8.
+inline int backward_waves(size_t x_elem_bytes, int waves) { return (x_elem_bytes == 4 || waves == 8) ? 8 : 16; }
+int backward_blocks(int64_t rows, int32_t D, size_t x_elem_bytes) {
+    const int waves = norm_waves(D), per = backward_waves(x_elem_bytes, waves), groups = per / waves;
+    const int64_t per_block = (int64_t)groups * kRowsPer;
+    const int64_t blocks = (rows + per_block - 1) / per_block;
+    const int64_t most = 256 * (16 / per);
+    return (int)(blocks < most ? blocks : most);
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; }
@@ -324,12 +381,6 @@ int check_norm(int64_t rows, int64_t cols, int dt_a, int dt_b) {
     for (int dt : {dt_a, dt_b})
         if (dt != SRU_AMD_F32 && dt != SRU_AMD_F16 && dt != SRU_AMD_BF16) return SRU_AMD_ERR_BAD_DTYPE;
     return SRU_AMD_OK;
-}
-
-// wavefronts per row: 8 features per lane
-inline int norm_waves(int32_t D) {
-    const int need = (D + kPass - 1) / kPass;
-    return need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
 }
 
 template <typename TI, typename TO>
@@ -354,11 +405,13 @@ hipError_t launch_norm_backward(const void *x, const float *gamma, const float *
     TD *di = static_cast<TD *>(dx);
     void *args[] = {&xi, &gamma, &mean, &rstd, &gi, &di, &partial, &rows, &D};
     const int waves = norm_waves(D);
-    const void *k = waves == 1   ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 1>)
-                    : waves == 2 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 2>)
-                    : waves == 4 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 4>)
-                                 : reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 8>);
-    return hipLaunchKernel(k, dim3(norm_blocks(rows)), dim3(kLanes * waves), args, 0, st);
+    constexpr int PER = sizeof(TI) == 4 ? 8 : 16;   // backward_waves()
+    const void *k = waves == 1   ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 1, PER>)
+                    : waves == 2 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 2, PER / 2>)
+                    : waves == 4 ? reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 4, PER / 4>)
+                                 : reinterpret_cast<const void *>(layer_norm_backward<TI, TG, TD, 8, 1>);
+    return hipLaunchKernel(k, dim3(backward_blocks(rows, D, sizeof(TI))), dim3(kLanes * backward_waves(sizeof(TI), waves)),
+                           args, 0, st);
 }
 
 // run F<A, B>(...) for the two runtime dtypes
@@ -400,8 +453,8 @@ int sru_amd_layer_norm_forward(int64_t rows, int64_t cols, const void *x, int x_
 
 size_t sru_amd_layer_norm_backward_workspace_bytes(int64_t rows, int64_t cols) {
     if (check_norm(rows, cols, SRU_AMD_F32, SRU_AMD_F32) != SRU_AMD_OK) return 0;
-    // one float row pair per workgroup of the backward kernel, then the slabs of the two-launch sum
-    return (size_t)norm_blocks(rows) * 2 * (size_t)cols * sizeof(float) + (size_t)kSlabs * 2 * (size_t)cols * sizeof(double);
+    // one float row pair per workgroup of the backward kernel (the larger of the two launch shapes)
+    return (size_t)backward_blocks(rows, (int32_t)cols, 4) * 2 * (size_t)cols * sizeof(float);
 }
 
 int sru_amd_layer_norm_backward(int64_t rows, int64_t cols, const void *x, int x_dtype, const float *weight,
@@ -424,26 +477,11 @@ int sru_amd_layer_norm_backward(int64_t rows, int64_t cols, const void *x, int x
         : x_dtype == SRU_AMD_F16 ? backward_by_grad<half_bits>(y_dtype, x, weight, mean, rstd, grad_y, grad_x, partial, rows, D, st)
                                  : backward_by_grad<bf16_bits>(y_dtype, x, weight, mean, rstd, grad_y, grad_x, partial, rows, D, st);
     if (err != hipSuccess) return SRU_AMD_ERR_LAUNCH;
-    int32_t nrows = norm_blocks(rows), width = 2 * D;
+    int32_t nrows = backward_blocks(rows, D, x_dtype == SRU_AMD_F32 ? 4 : 2), width = 2 * D;
     const float *src = partial;
-    const dim3 columns((width + kLanes - 1) / kLanes), threads(kLanes * kRowSlices);
-    if (nrows <= 4 * kSlabs) {
-        int32_t chunk = nrows;
-        void *args[] = {&src, &grad_weight, &nrows, &width, &chunk};
-        return hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows<float, float>), columns, threads, args, 0, st) ==
-                       hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
-    }
-    double *slabs = reinterpret_cast<double *>(partial + (size_t)nrows * width);
-    int32_t chunk = (nrows + kSlabs - 1) / kSlabs;
-    void *first[] = {&src, &slabs, &nrows, &width, &chunk};
-    if (hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows<float, double>), dim3(columns.x, kSlabs), threads, first,
-                        0, st) != hipSuccess)
-        return SRU_AMD_ERR_LAUNCH;
-    const double *mid = slabs;
-    int32_t nslabs = kSlabs, all = kSlabs;
-    void *second[] = {&mid, &grad_weight, &nslabs, &width, &all};
-    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows<double, float>), columns, threads, second, 0, st) ==
-                   hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
+    void *args[] = {&src, &grad_weight, &nrows, &width};
+    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_rows), dim3((width + kLanes - 1) / kLanes),
+                           dim3(kLanes * kRowSlices), args, 0, st) == hipSuccess ? SRU_AMD_OK : SRU_AMD_ERR_LAUNCH;
 }
 
 }  // extern "C"

@@ -334,6 +334,7 @@ struct FwdParams {
     int64_t L, B, ncols;  // ncols = B * D'
     int32_t d, Dp;        // hidden per direction, D' = dirs * d
     int32_t act, custom;  // act: host-side kernel selection and the general kernels; custom: general kernels
+    int32_t x_float;      // host-side kernel selection: x is float next to 16-bit streams
 };
 
 struct BwdParams {
@@ -350,6 +351,7 @@ struct BwdParams {
     int64_t L, B, ncols;
     int32_t d, Dp;
     int32_t act, custom;
+    int32_t x_float;      // host-side kernel selection: x and grad_x are float next to 16-bit streams
 };
 
 // Every field of the parameter block is read at the top of a kernel. Left alone, the compiler
@@ -575,10 +577,13 @@ __device__ __forceinline__ LiveWindow live_window(const uint8_t *pad, int64_t pf
 // (Fast kernels only; TC equals the checkpoint interval. The two lambdas must be inlined at
 // every call site: a chunk that is passed by reference to a real function lives in scratch
 // memory instead of registers.)
-template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
+// TX: element type of x (the skip term when SKIP == 1): T, or float next to 16-bit streams (under
+// autocast the layer's input stays float while U comes out of the projection in 16 bits).
+template <typename T, int K, int SKIP, int MODE, int COLS, int TC, typename TX = T>
 __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward_scan_chunked(const FwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
     static_assert(TC == kCkptInterval, "a chunk is one checkpoint interval");
+    static_assert(sizeof(TX) == sizeof(T) || (sizeof(TX) == 4 && SKIP == 1), "a float x next to 16-bit streams");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, KEEP_C = (MODE & kKeepC) != 0;
     constexpr bool CKPT = (MODE & kCkpt) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
@@ -592,7 +597,8 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
     constexpr int kPadRegs = PAD_BY_LANE ? 1 : TC;
     fetch_params_early(p);
     using SU = Stream<T, K, COLS, PAIR>;   // U: K elements per column
-    using S1 = Stream<T, 1, COLS, PAIR>;   // x, h, c: one element per column
+    using S1 = Stream<T, 1, COLS, PAIR>;   // h, c: one element per column
+    using SX = Stream<TX, 1, COLS, PAIR && sizeof(TX) == 2>;   // x (a float x needs no lane pairing)
     using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c: two elements per column
     // the wavefront's index in the launch (scalar), and the lane's in the wavefront
     const uint32_t wg = blockIdx.x * (blockDim.x / kBlock) + (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kBlock));
@@ -630,14 +636,14 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
     const int64_t pf = (flip ? (L - 1) : 0) * p.B + col / Dp;
     const int64_t ps = flip ? -p.B : p.B;
     const T *ubase = static_cast<const T *>(p.u);
-    const T *xbase = static_cast<const T *>(p.x);
+    const TX *xbase = static_cast<const TX *>(p.x);
     T *hbase = static_cast<T *>(p.h);
     T *cbase = static_cast<T *>(p.c);
     const T *vbase = static_cast<const T *>(p.wc);   // CUSTOM only
 
     struct Chunk {
         typename SU::G u[TC];
-        typename S1::G x[TC];
+        typename SX::G x[TC];
         typename SV::G w[CUSTOM ? TC : 1];
         uint32_t pad[kPadRegs];  // padding flags of the chunk, see load_chunk
     };
@@ -649,7 +655,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
             if (i < n) {
                 const int64_t e = ef + (s0 + i) * es;
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
-                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
+                if (SKIP == 1) k.x[i] = SX::template load<NTL>(xbase + e, lane, q);
                 if constexpr (CUSTOM) k.w[i] = SV::template load<NTL>(vbase + e * 2, lane, q);
                 if (!PAD_BY_LANE) k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
             }
@@ -671,7 +677,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
                 const uint32_t keep = 0u - (uint32_t)(flag != 0);   // all ones at a padded step
                 float hv[COLS], cv[COLS], uu[COLS * K], xx[COLS] = {};
                 SU::unpack(k.u[i], q, uu);
-                if (SKIP == 1) S1::unpack(k.x[i], q, xx);
+                if (SKIP == 1) SX::unpack(k.x[i], q, xx);
                 float ww[COLS * 2] = {};
                 if constexpr (CUSTOM) SV::unpack(k.w[i], q, ww);
 #pragma unroll
@@ -959,16 +965,19 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
 // recurrence over the same registers. Loads of the next chunk are issued before the
 // arithmetic of the current one. Per cell: reads U (k), x, grad_h and 4/TC bytes of
 // checkpoint; writes grad_u (k), grad_x.
-template <typename T, int K, int SKIP, int MODE, int COLS, int TC>
+// TX: element type of x and grad_x, see forward_scan_chunked.
+template <typename T, int K, int SKIP, int MODE, int COLS, int TC, typename TX = T>
 __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backward_scan_ckpt(const BwdParams p) {
     static_assert((MODE & kGeneral) == 0, "fast kernels only");
+    static_assert(sizeof(TX) == sizeof(T) || (sizeof(TX) == 4 && SKIP == 1), "a float x next to 16-bit streams");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     constexpr bool HAS_PAD = (MODE & kHasPad) != 0, PAIR = (MODE & kPair) != 0, UNI = (MODE & kUniform) != 0;
     // (forward_scan_chunked fetches the flags of a chunk with one load; here, where every flag
     // is needed twice, that measured 0-3 % slower, so the flags stay one load per step)
     constexpr bool TANH = (MODE & kTanh) != 0, CUSTOM = (MODE & kCustom) != 0;
     using SU = Stream<T, K, COLS, PAIR>;   // U, grad_u: K elements per column
-    using S1 = Stream<T, 1, COLS, PAIR>;   // x, grad_h, grad_x: one element per column
+    using S1 = Stream<T, 1, COLS, PAIR>;   // grad_h: one element per column
+    using SX = Stream<TX, 1, COLS, PAIR && sizeof(TX) == 2>;   // x, grad_x
     using SV = Stream<T, 2, COLS, PAIR>;   // a per-step weight_c and its gradient: two elements per column
     fetch_params_early(p);
     // the wavefront's index in the launch (scalar), and the lane's in the wavefront
@@ -1008,16 +1017,16 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
     const int64_t pf = (flip ? (L - 1) : 0) * p.B + col / Dp;
     const int64_t ps = flip ? -p.B : p.B;
     const T *ubase = static_cast<const T *>(p.u);
-    const T *xbase = static_cast<const T *>(p.x);
+    const TX *xbase = static_cast<const TX *>(p.x);
     const T *ghbase = static_cast<const T *>(p.gh);
     T *gubase = static_cast<T *>(p.gu);
-    T *gxbase = static_cast<T *>(p.gx);
+    TX *gxbase = static_cast<TX *>(p.gx);
     const T *vbase = static_cast<const T *>(p.wc);   // CUSTOM only
     T *gvbase = static_cast<T *>(p.gwc_steps);
 
     struct Chunk {
         typename SU::G u[TC];
-        typename S1::G x[TC];
+        typename SX::G x[TC];
         typename S1::G gh[TC];
         typename SV::G w[CUSTOM ? TC : 1];
         uint32_t pad[TC];    // padding flags of the chunk's steps
@@ -1032,7 +1041,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
             if (i < n) {
                 const int64_t e = ef + (s0 + i) * es;
                 k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
-                if (SKIP == 1) k.x[i] = S1::template load<NTL>(xbase + e, lane, q);
+                if (SKIP == 1) k.x[i] = SX::template load<NTL>(xbase + e, lane, q);
                 k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
                 if constexpr (CUSTOM) k.w[i] = SV::template load<NTL>(vbase + e * 2, lane, q);
                 k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
@@ -1096,7 +1105,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
             if (i < n) {
                 const bool padded = k.pad[i] != 0;
                 float gu[COLS * K], gx[COLS], xx[COLS] = {}, ghs[COLS];
-                if (SKIP == 1) S1::unpack(k.x[i], q, xx);
+                if (SKIP == 1) SX::unpack(k.x[i], q, xx);
                 S1::unpack(k.gh[i], q, ghs);
                 float ww[COLS * 2] = {}, gv[COLS * 2];
                 if constexpr (CUSTOM) SV::unpack(k.w[i], q, ww);
@@ -1131,7 +1140,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
                 }
                 const int64_t e = ef + (s0 + i) * es;
                 SU::template store<NTS>(gubase + e * K, lane, q, gu);
-                if (SKIP == 1) S1::template store<NTS>(gxbase + e, lane, q, gx);
+                if (SKIP == 1) SX::template store<NTS>(gxbase + e, lane, q, gx);
                 if constexpr (CUSTOM) SV::template store<NTS>(gvbase + e * 2, lane, q, gv);
             }
         }
@@ -1150,7 +1159,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
         for (int64_t s = from; s < to; ++s) {
             const int64_t e = ef + s * es;
             SU::template store<NTS>(gubase + e * K, lane, q, zu);
-            if (SKIP == 1) S1::template store<NTS>(gxbase + e, lane, q, z1);
+            if (SKIP == 1) SX::template store<NTS>(gxbase + e, lane, q, z1);
             if constexpr (CUSTOM) SV::template store<NTS>(gvbase + e * 2, lane, q, zv);
         }
     };

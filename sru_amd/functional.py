@@ -16,7 +16,11 @@ What moves into the kernels compared with the reference's Python:
     kernels write every cell.
 
 The large streams (U, x, h, c and their gradients) are consumed in the dtype of
-`u` (float32, float16 or bfloat16); state and arithmetic are float32.
+`u` (float32, float16 or bfloat16); state and arithmetic are float32. A float32 x
+beside a 16-bit U (the layer's input under autocast, which the reference keeps in
+float32 too, sru/ops.py:121) is read as it is, and grad_x comes back in float32,
+wherever the kernels take it (plain layer: vector weight_c, identity activation, even
+d); elsewhere x is rounded to u's dtype first. A float64 U is computed in float32.
 """
 from typing import Optional, Tuple
 
@@ -55,7 +59,7 @@ class _Problem:
     immutable and shared: `_problem()` keeps one per distinct (shape, dtype, flags)."""
 
     def __init__(self, dtype, x_dim, length, batch, u_numel, u_last, is_custom, d_out,
-                 bidirectional, has_skip_term, activation_type, checkpoint_state):
+                 bidirectional, has_skip_term, activation_type, checkpoint_state, x_is_float, state_kept):
         if dtype not in _DTYPES:
             raise ValueError(f"U must be float32, float16 or bfloat16, not {dtype}")
         if x_dim not in (2, 3):
@@ -80,10 +84,16 @@ class _Problem:
         # 16-bit streams need an even d for that; a per-step weight_c must not come with tanh.
         ok = (dtype == torch.float32 or d_out % 2 == 0) and not (self.is_custom and activation_type != 0)
         self.checkpointed = bool(checkpoint_state and ok and not (self.skip_type == 0 and self.k == 4))
+        # A float32 x beside 16-bit streams (the layer's input under autocast) is read as it is by
+        # the chunked kernels of the plain layer; everywhere else x is rounded to the stream dtype.
+        self.x_float = bool(x_is_float and dtype != torch.float32 and self.skip_type == 1 and not self.is_custom
+                            and activation_type == 0 and d_out % 2 == 0 and (self.checkpointed or not state_kept))
+        self.x_dtype = torch.float32 if self.x_float else dtype
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
                                 activation_type, self.skip_type, self.is_custom,
                                 _DTYPES[dtype],
-                                _lib.STATE_INTERVAL if self.checkpointed else 1)
+                                _lib.STATE_INTERVAL if self.checkpointed else 1,
+                                _lib.X_F32 if self.x_float else _lib.X_AS_STREAMS)
         lib = _lib.load()
         self.state_rows = lib.sru_amd_state_bytes(ctypes.byref(self.shape)) // (4 * self.batch * self.Dp) \
             if self.checkpointed else self.length
@@ -98,14 +108,16 @@ _problem_cached = functools.lru_cache(maxsize=256)(_Problem)
 
 
 def _problem(u: Tensor, x: Tensor, weight_c: Tensor, d_out: int, bidirectional: bool,
-             has_skip_term: bool, activation_type: int, checkpoint_state: bool = False) -> _Problem:
+             has_skip_term: bool, activation_type: int, checkpoint_state: bool = False,
+             state_kept: bool = True) -> _Problem:
     if not u.is_cuda:
         raise RuntimeError("the SRU recurrence kernels need device tensors (got a CPU tensor)")
     if x.dim() not in (2, 3):
         raise ValueError("x must be 2 or 3 dimensional")
     return _problem_cached(u.dtype, x.dim(), x.size(0) if x.dim() == 3 else 1, x.size(-2), u.numel(),
                            u.size(-1), 1 if weight_c.dim() > 1 else 0, d_out, bool(bidirectional),
-                           bool(has_skip_term), int(activation_type), bool(checkpoint_state))
+                           bool(has_skip_term), int(activation_type), bool(checkpoint_state),
+                           x.dtype == torch.float32, bool(state_kept))
 
 
 def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad):
@@ -113,7 +125,7 @@ def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, m
     u_ = _aligned(u, 16)
     x_ = None
     if pb.skip_type == 1:
-        x_ = _aligned(x if x.dtype == pb.dtype else x.to(pb.dtype), 4)
+        x_ = _aligned(x if x.dtype == pb.x_dtype else x.to(pb.x_dtype), 4)
         if x_.numel() != pb.length * pb.batch * pb.Dp:
             raise ValueError("x must have length*batch*output_size elements when it is the skip term")
     if pb.is_custom:
@@ -185,7 +197,7 @@ def elementwise_recurrence_forward(
     out_dtype = u.dtype
     if u.dtype != _kernel_dtype(u):
         u = u.to(_kernel_dtype(u))
-    pb = _problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type)
+    pb = _problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type, state_kept=keep_c)
     prepared = _prepare_inputs(pb, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad)
     h, c, c_last = _run_forward(pb, *prepared, keep_c=keep_c)
     last_hidden = c_last if out_dtype == torch.float32 else c_last.to(out_dtype)

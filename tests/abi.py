@@ -18,22 +18,25 @@ def p(t):
 class DeviceProblem:
     """Device copies of a Case in stream dtype `dt`; float32 for the small tensors."""
 
-    def __init__(self, case, dt="f32", device="cuda:0", checkpointed=False):
+    def __init__(self, case, dt="f32", device="cuda:0", checkpointed=False, x_f32=False):
         """checkpointed: keep float state checkpoints between forward and backward
-        (shape.state_interval = SRU_AMD_STATE_INTERVAL) instead of the state after every step."""
-        self.case, self.dt, self.checkpointed = case, dt, checkpointed
+        (shape.state_interval = SRU_AMD_STATE_INTERVAL) instead of the state after every step.
+        x_f32: x and grad_x are float32 beside 16-bit streams (shape.x_dtype = SRU_AMD_X_F32)."""
+        self.case, self.dt, self.checkpointed, self.x_f32 = case, dt, checkpointed, x_f32
         tdt = TORCH_DT[dt]
         dev = torch.device(device)
         big = lambda a: torch.tensor(a, dtype=tdt, device=dev).contiguous()
         small = lambda a: None if a is None else torch.tensor(a, dtype=torch.float32, device=dev).contiguous()
         c = case
         self.U, self.x, self.gh = big(c.U), big(c.x), big(c.gh)
+        if x_f32:
+            self.x = torch.tensor(c.x, dtype=torch.float32, device=dev).contiguous()
         self.wc = big(c.wc) if c.custom else small(c.wc)
         self.bias, self.c0, self.gl, self.mask_c = small(c.bias), small(c.c0), small(c.gl), small(c.mask_c)
         self.scale = torch.tensor([c.scale], dtype=torch.float32, device=dev)
         self.pad = None if c.pad is None else torch.tensor(c.pad, dtype=torch.bool, device=dev).view(torch.uint8)
         self.shape = _lib.Shape(c.L, c.B, c.d, c.dirs, c.k, c.act, c.skip_type, c.custom, CODE[dt],
-                                _lib.STATE_INTERVAL if checkpointed else 1)
+                                _lib.STATE_INTERVAL if checkpointed else 1, _lib.X_F32 if x_f32 else _lib.X_AS_STREAMS)
         self.dev, self.tdt = dev, tdt
 
     def rounded_case(self):
@@ -71,7 +74,7 @@ class DeviceProblem:
         mk = (lambda *s, dtype: torch.full(s, float("nan"), dtype=dtype, device=self.dev)) if poison else \
             (lambda *s, dtype: torch.empty(s, dtype=dtype, device=self.dev))
         self.gu = mk(c.L, c.B, c.Dp * c.k, dtype=self.tdt)
-        self.gx = mk(c.L, c.B, c.Dp, dtype=self.tdt) if c.skip_type == 1 else None
+        self.gx = mk(c.L, c.B, c.Dp, dtype=torch.float32 if self.x_f32 else self.tdt) if c.skip_type == 1 else None
         self.gwc = mk(c.L, c.B, c.Dp * 2, dtype=self.tdt) if c.custom else mk(2 * c.Dp, dtype=torch.float32)
         self.gb = mk(2 * c.Dp, dtype=torch.float32)
         self.gi = mk(c.B, c.Dp, dtype=torch.float32)

@@ -25,12 +25,12 @@ def test_exports_every_declared_symbol():
 def test_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.Shape) == 56
     assert _lib.Shape.dirs.offset == 24 and _lib.Shape.dtype.offset == 44
-    assert _lib.Shape.state_interval.offset == 48
+    assert _lib.Shape.state_interval.offset == 48 and _lib.Shape.x_dtype.offset == 52
 
 
 def _shape(**kw):
     base = dict(length=4, batch=2, hidden=8, dirs=2, k=3, activation_type=0, skip_type=1,
-                is_custom=0, dtype=0, state_interval=0)
+                is_custom=0, dtype=0, state_interval=0, x_dtype=0)
     base.update(kw)
     return _lib.Shape(*[base[f[0]] for f in _lib.Shape._fields_])
 
@@ -46,6 +46,9 @@ FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
     (dict(state_interval=4), 3),
     (dict(state_interval=8, is_custom=1, activation_type=1), 3), (dict(state_interval=8, skip_type=0, k=4), 3),
     (dict(state_interval=8, dtype=2, hidden=7), 3), (dict(state_interval=8, dtype=1, hidden=1), 3),
+    # a float x beside 16-bit streams: plain layer only, even hidden; with float streams the field changes nothing
+    (dict(x_dtype=2), 4), (dict(x_dtype=1, dtype=2, state_interval=8, is_custom=1), 3),
+    (dict(x_dtype=1, dtype=1, state_interval=8, activation_type=1), 3), (dict(x_dtype=1, dtype=2, hidden=7), 3),
 ])
 def test_forward_rejects_bad_shapes(kw, code):
     lib = _lib.load()
@@ -89,6 +92,17 @@ def test_null_and_misaligned_pointers_and_workspace():
         assert lib.sru_amd_backward(ctypes.byref(s), *bad, need, None) == 1, required
 
 
+def test_float_x_beside_16bit_streams_needs_checkpoints_or_no_state():
+    lib = _lib.load()
+    s = _shape(dtype=2, x_dtype=1, state_interval=1)
+    assert lib.sru_amd_forward(ctypes.byref(s), *([FAKE] * 11), None) == 3       # c given, state after every step
+    assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), 1 << 20, None) == 3
+    s = _shape(dtype=2, x_dtype=1, state_interval=8)
+    bad = [FAKE] * 11
+    bad[1] = ctypes.c_void_p(0x1002)             # the float x must be 4-byte aligned
+    assert lib.sru_amd_forward(ctypes.byref(s), *bad, None) == 5
+
+
 def test_static_backward_checks_sizes_before_anything_else():
     # the allocation-free entry point refuses more columns than its built-in array holds
     lib = _lib.load()
@@ -109,9 +123,10 @@ def test_layer_norm_entry_points_validate_before_launching():
     assert fwd(4, 64, x=None) == 1
     assert fwd(4, 64, x=ctypes.c_void_p(0x1004)) == 5
     need = lib.sru_amd_layer_norm_backward_workspace_bytes(4, 64)
-    slabs = 16 * 2 * 8    # bytes per feature of the second stage of the sum over workgroups
-    assert need == 2 * 2 * 64 * 4 + slabs * 64 and lib.sru_amd_layer_norm_backward_workspace_bytes(4, 12) == 0
-    assert lib.sru_amd_layer_norm_backward_workspace_bytes(10 ** 6, 1024) == 1024 * 2 * 1024 * 4 + slabs * 1024
+    # one (2, cols) float row per workgroup of the backward kernel: one workgroup here, 512 at most
+    assert need == 2 * 64 * 4 and lib.sru_amd_layer_norm_backward_workspace_bytes(4, 12) == 0
+    assert lib.sru_amd_layer_norm_backward_workspace_bytes(16384, 2048) == 512 * 2 * 2048 * 4
+    assert lib.sru_amd_layer_norm_backward_workspace_bytes(10 ** 6, 4096) == 512 * 2 * 4096 * 4   # 8 wavefronts per row
     gw = ctypes.c_void_p(0x2000)
     gb = ctypes.c_void_p(0x2000 + 64 * 4)
     bwd = lambda ws, nbytes, gbias=gb: lib.sru_amd_layer_norm_backward(

@@ -159,3 +159,44 @@ def test_u_view_at_an_unaligned_offset_is_copied_not_refused():
         h.float().sum().backward()
         outs.append((h.detach(), u.grad))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+def test_float32_x_beside_bf16_u_is_not_rounded():
+    """Under autocast the layer's input stays float32 while U is 16-bit: x goes to the kernels as it
+    is (no cast pass, no rounding) and grad_x comes back in float32. Checked against a run whose x was
+    rounded to bfloat16 first (must differ, and by no more than that rounding) and against the float64
+    restatement fed the same values."""
+    from sru_amd import ElementwiseRecurrence
+    from sru_amd.functional import _problem
+    c = Case(L=24, B=4, d=128, dirs=2, seed=48, scale=1.7, pad="right")
+    dev = "cuda:0"
+    t = lambda a, dt=torch.float32, rg=True: torch.tensor(a, dtype=dt, device=dev, requires_grad=rg)
+    u = t(c.U, torch.bfloat16)
+    x = t(c.x)
+    wc, bias, c0 = t(c.wc), t(c.bias), t(c.c0)
+    sx = torch.tensor([c.scale], device=dev)
+    pad = torch.tensor(c.pad, device=dev)
+    assert _problem(u, x, wc, c.d, True, True, 0, checkpoint_state=True).x_float
+    h, last = ElementwiseRecurrence.apply(u, x, wc, bias, c0, 0, c.d, True, True, sx, None, pad)
+    gh = torch.tensor(c.gh, dtype=torch.bfloat16, device=dev)
+    (h * gh).sum().backward()
+    assert h.dtype == torch.bfloat16 and x.grad.dtype == torch.float32
+    # float64 restatement on the values the kernels saw
+    import copy
+    c64 = copy.copy(c)
+    c64.U, c64.gh = u.detach().double().cpu().numpy(), gh.double().cpu().numpy()
+    c64.x = x.detach().double().cpu().numpy()
+    c64.gl = np.zeros_like(c.gl)
+    for n in ("wc", "bias", "c0"):
+        setattr(c64, n, getattr(c, n).astype(np.float32).astype(np.float64))
+    c64.scale = float(np.float32(c.scale))
+    h_ref, _, g_ref = _apply(st.recurrence, c64, "cpu", torch.float64)
+    assert np.abs(h.detach().double().cpu().numpy() - h_ref).max() <= 2e-2 * max(1.0, np.abs(h_ref).max())
+    gx = x.grad.double().cpu().numpy()
+    assert (np.abs(gx - g_ref[1]) / np.maximum(1.0, np.abs(g_ref[1]))).max() <= 2e-2
+    # against the rounded-x run: different, but only by the rounding of x
+    x16 = t(c.x, torch.bfloat16)
+    h16, _ = ElementwiseRecurrence.apply(u.detach(), x16, wc.detach(), bias.detach(), c0.detach(), 0, c.d, True, True,
+                                         sx, None, pad)
+    assert not torch.equal(h16, h.detach())
+    assert float((h16.float() - h.detach().float()).abs().max()) <= 2e-2 * max(1.0, float(h.detach().float().abs().max()))

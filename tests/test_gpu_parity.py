@@ -49,10 +49,11 @@ def _cell_err(a, b):
     return float(d.max()) if d.size else 0.0
 
 
-def check_against_oracle(case, dt="f32", keep_c=True, checkpointed=False):
+def check_against_oracle(case, dt="f32", keep_c=True, checkpointed=False, x_f32=False):
     """checkpointed: the state travels from forward to backward as float checkpoints every
-    SRU_AMD_STATE_INTERVAL steps and the backward kernel rebuilds the rest."""
-    dp = DeviceProblem(case, dt, checkpointed=checkpointed)
+    SRU_AMD_STATE_INTERVAL steps and the backward kernel rebuilds the rest.
+    x_f32: x and grad_x are float32 beside the 16-bit streams."""
+    dp = DeviceProblem(case, dt, checkpointed=checkpointed, x_f32=x_f32)
     rc = dp.rounded_case()
     h, c, c_last = dp.forward(keep_c=keep_c)
     h_ref, c_ref, cl_ref = so.forward(*rc.fwd_args(), **rc.kw())
@@ -329,3 +330,23 @@ def test_long_right_padded_rows_forward_only_and_training(dt):
     check_against_oracle(c, dt, keep_c=False)
     check_against_oracle(c, dt, checkpointed=True)
 
+
+
+FLOAT_X = [
+    dict(L=21, B=3, d=64, dirs=2, scale=1.7),                             # lane pairs, wave-uniform
+    dict(L=40, B=4, d=70, dirs=2, pad="right", scale=1.3, mask_c=True),   # lane pairs, wavefronts straddle rows
+    dict(L=17, B=2, d=6, pad="random"),                                   # less than a wavefront
+    dict(L=19, B=64, d=1024, dirs=2, pad="right", scale=1.7),             # two columns per lane (131 072 columns)
+    dict(L=12, B=1100, d=70, dirs=2, pad="random", scale=0.8),            # two columns per lane, straddling rows
+]
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("cfg", FLOAT_X, ids=_ids)
+def test_float_x_beside_16bit_streams(cfg, dt):
+    """x stays float32 while U, h and grad_h are 16-bit (shape.x_dtype = SRU_AMD_X_F32): training with
+    checkpoints, and inference without a state store. Same bounds as the 16-bit runs; grad_x comes
+    back in float32 and is held per cell."""
+    c = Case(seed=47, **cfg)
+    check_against_oracle(c, dt, checkpointed=True, x_f32=True)
+    check_against_oracle(c, dt, keep_c=False, x_f32=True)
