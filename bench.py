@@ -174,20 +174,21 @@ def run_stack(args):
         (h.float() * probe).sum().backward()
         model.zero_grad(set_to_none=True)
 
-    if args.graph:      # record the forward once, replay it per step (launch-bound shapes)
-        if not forward_only:
-            sys.exit("bench.py: --graph records the forward-only stack (stack1)")
-        model.eval()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            for _ in range(3):
-                step()
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            step()
-        step = graph.replay
+    if args.graph:      # record once with sru_amd.graphed, replay per step (launch-bound shapes)
+        if forward_only:
+            model.eval()
+            with torch.no_grad():
+                fast = sru_amd.graphed(model, x, autocast_dtype=amp)
+
+            def step():
+                return fast(x)
+        else:
+            fast = sru_amd.graphed(model, x, mask_pad=mask_pad, autocast_dtype=amp)
+
+            def step():
+                h, _ = fast(x, mask_pad=mask_pad)
+                (h.float() * probe).sum().backward()
+                model.zero_grad(set_to_none=True)
 
     for _ in range(args.warmup):
         step()

@@ -17,7 +17,7 @@ from torch import Tensor
 from torch.autograd import Function
 
 from . import _lib
-from .functional import _DTYPES, _aligned, _f32, _ptr
+from .functional import _DTYPES, _aligned, _f32, _on_device, _ptr
 
 
 def supported(x: Tensor) -> bool:
@@ -35,8 +35,7 @@ class LayerNormFunction(Function):
         y = torch.empty(x_.shape, dtype=out_dtype, device=x.device)
         mean = torch.empty(rows, dtype=torch.float32, device=x.device)
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
-        with torch.cuda.device(x.device):
-            stream = ctypes.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)
+        with _on_device(x.device) as stream:
             rc = _lib.load().sru_amd_layer_norm_forward(rows, D, _ptr(x_), _DTYPES[x_.dtype], _ptr(w_), _ptr(b_),
                                                         ctypes.c_float(eps), _ptr(y), _DTYPES[out_dtype],
                                                         _ptr(mean), _ptr(rstd), stream)
@@ -56,8 +55,7 @@ class LayerNormFunction(Function):
         lib = _lib.load()
         nbytes = lib.sru_amd_layer_norm_backward_workspace_bytes(rows, D)
         workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=x_.device)
-        with torch.cuda.device(x_.device):
-            stream = ctypes.c_void_p(torch.cuda.current_stream(x_.device).cuda_stream)
+        with _on_device(x_.device) as stream:
             rc = lib.sru_amd_layer_norm_backward(rows, D, _ptr(x_), _DTYPES[x_.dtype], _ptr(w_), _ptr(mean),
                                                  _ptr(rstd), _ptr(gy), _DTYPES[gy.dtype], _ptr(grad_x),
                                                  _ptr(grad_wb[0]), _ptr(grad_wb[1]), _ptr(workspace),
