@@ -309,6 +309,9 @@ def main():
                     help="with a stack workload: use torch.nn.LayerNorm's kernels instead of this package's")
     ap.add_argument("--shape", default=None, metavar="L,B,d,dirs",
                     help="side measurement at another shape (k=3 forward + backward, no padding); replaces --workload")
+    ap.add_argument("--x-f32", action="store_true",
+                    help="side measurement with 16-bit streams: x and grad_x stay float32 (shape.x_dtype = "
+                         "SRU_AMD_X_F32), as the layer's input does under autocast")
     ap.add_argument("--fixed-length", type=int, default=0,
                     help="side measurement with a padded workload: every sequence has this length (default: "
                          "lengths uniform in [L/4, L])")
@@ -354,9 +357,14 @@ def main():
         name += " no skip term"
     if custom:
         name += " per-step weight_c"
+    x_f32 = args.x_f32 and es == 2 and use_x
+    if x_f32:
+        name += " float32 x"
     shape = _lib.Shape(L, B, d, dirs, k, 1 if args.tanh else 0,
                        0 if args.no_skip else (1 if k == 3 else 2), 1 if custom else 0, CODE[args.dtype],
-                       _lib.STATE_INTERVAL if ckpt else 1)
+                       _lib.STATE_INTERVAL if ckpt else 1, _lib.X_F32 if x_f32 else _lib.X_AS_STREAMS)
+    xdt = torch.float32 if x_f32 else tdt
+    xs = 4 if x_f32 else es   # bytes per element of x and grad_x
     state_rows = lib.sru_amd_state_bytes(ctypes.byref(shape)) // (B * Dp * (4 if ckpt else DT_BYTES[args.dtype]))
 
     g = torch.Generator(device=dev).manual_seed(1234)
@@ -364,12 +372,12 @@ def main():
     for _ in range(args.sets):
         s = dict(
             U=torch.randn(L, B, Dp * k, device=dev, generator=g).to(tdt),
-            x=torch.randn(L, B, Dp, device=dev, generator=g).to(tdt),
+            x=torch.randn(L, B, Dp, device=dev, generator=g).to(xdt),
             gh=torch.randn(L, B, Dp, device=dev, generator=g).to(tdt),
             h=torch.empty(L, B, Dp, device=dev, dtype=tdt),
             c=torch.empty(state_rows, B, Dp, device=dev, dtype=torch.float32 if ckpt else tdt),
             gu=torch.empty(L, B, Dp * k, device=dev, dtype=tdt),
-            gx=torch.empty(L, B, Dp, device=dev, dtype=tdt),
+            gx=torch.empty(L, B, Dp, device=dev, dtype=xdt),
         )
         sets.append(s)
     wc = (torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1) * 1.5 ** 0.5
@@ -500,8 +508,8 @@ def main():
     # x, c, grad_h and writes grad_u (k), grad_x.
     # (a per-step weight_c is one more stream of 2 elements per cell: read by both passes, its
     # gradient written by the backward pass)
-    fwd_bytes = (k + (1 if use_x else 0) + (1 if fwd_only else 2) + (2 if custom else 0)) * es * cells
-    bwd_bytes = (2 * k + (2 if use_x else 0) + 2 + (4 if custom else 0)) * es * cells
+    fwd_bytes = (k + (1 if fwd_only else 2) + (2 if custom else 0)) * es * cells + (xs * cells if use_x else 0)
+    bwd_bytes = (2 * k + 2 + (4 if custom else 0)) * es * cells + (2 * xs * cells if use_x else 0)
     # What the selected kernels are built to move: with checkpoints the per-step state (es bytes per
     # cell each way) shrinks to one float per 8 steps.
     state_bytes = (4 * cells // 8) if ckpt else es * cells
@@ -516,10 +524,10 @@ def main():
         uniform = d % (64 * cols) == 0 and not lane_pairs and not (custom and args.tanh)
         live_f = walked if uniform else 1.0
         live_b = walked if uniform and ckpt else 1.0   # (the state-after-every-step backward kernel walks every step)
-    fwd_in = (k + (1 if use_x else 0) + (2 if custom else 0)) * es * cells
-    bwd_in = (k + (1 if use_x else 0) + 1 + (2 if custom else 0)) * es * cells + state_bytes
+    fwd_in = (k + (2 if custom else 0)) * es * cells + (xs * cells if use_x else 0)
+    bwd_in = (k + 1 + (2 if custom else 0)) * es * cells + (xs * cells if use_x else 0) + state_bytes
     fwd_moved = int(fwd_in * live_f) + es * cells + (0 if fwd_only else state_bytes)
-    bwd_moved = int(bwd_in * live_b) + (k + (1 if use_x else 0) + (2 if custom else 0)) * es * cells
+    bwd_moved = int(bwd_in * live_b) + (k + (2 if custom else 0)) * es * cells + (xs * cells if use_x else 0)
     if fwd_only:
         bwd_us = float("nan")
     bwd_gbs = bwd_bytes / (bwd_us * 1e-6) / 1e9
