@@ -24,17 +24,24 @@
  * Layouts (those of the reference)
  *   U        (L, B, D', k)      k innermost; D' = dirs * hidden
  *   x, h, c, grad_h, grad_x     (L, B, D')            (x, grad_x: see shape->x_dtype)
- *   weight_c (2, D') float, or, when is_custom, (L, B, D', 2) in `dtype`
- *   bias     (2, D') float
- *   c_init, mask_c, c_last, grad_last, grad_init   (B, D') float
+ *   weight_c (2, D') small, or, when is_custom, (L, B, D', 2) in `dtype`
+ *   bias     (2, D') small
+ *   c_init, mask_c, c_last, grad_last, grad_init   (B, D') small
  *   mask_pad (L, B) one byte per cell, non-zero = padded
- *   scale_x  one float on the device, or NULL for 1
+ *   scale_x  one small value on the device, or NULL for 1
  * `dtype` is the element type of the large streams U, x, h, c, grad_h, grad_u,
- * grad_x and of a per-step weight_c / its gradient. The recurrence state and all
- * arithmetic are float whatever `dtype` is.
+ * grad_x and of a per-step weight_c / its gradient. With SRU_AMD_F32, SRU_AMD_F16 and
+ * SRU_AMD_BF16 the recurrence state and all arithmetic are float, and so is every tensor
+ * marked "small" below. With SRU_AMD_F64 everything is double: the streams, the small
+ * tensors (weight_c, bias, c_init, mask_c, scale_x, c_last, grad_last, grad_wc, grad_bias,
+ * grad_init), the state and the arithmetic, as in the reference's double kernels
+ * (sru/csrc/sru_cuda_kernel.cu:845, AT_DISPATCH_FLOATING_TYPES_AND_HALF); the backward
+ * workspace doubles with it. The small tensors are therefore declared `void *`: float
+ * unless `dtype` is SRU_AMD_F64.
  *
  * Alignment (SRU_AMD_ERR_MISALIGNED otherwise)
- *   - float tensors: 4 bytes; U and grad_u with k = 4: four elements (one group);
+ *   - small tensors: their element size; U and grad_u with k = 4: four elements (one group; 16 bytes
+ *     are enough for double streams);
  *   - every stream: its element size; a per-step weight_c and its gradient: two elements;
  *   - 16-bit streams with state_interval == SRU_AMD_STATE_INTERVAL move two columns at a
  *     time: x, h, grad_h, grad_x 4 bytes; U and grad_u 4 bytes (k = 3) or 16 bytes (k = 4);
@@ -52,12 +59,13 @@
 extern "C" {
 #endif
 
-#define SRU_AMD_ABI_VERSION 5
+#define SRU_AMD_ABI_VERSION 6
 
 enum sru_amd_dtype {
     SRU_AMD_F32 = 0,
     SRU_AMD_F16 = 1,
-    SRU_AMD_BF16 = 2
+    SRU_AMD_BF16 = 2,
+    SRU_AMD_F64 = 3     /* double streams, small tensors, state and arithmetic; state_interval 0 / 1 only */
 };
 
 enum sru_amd_status {
@@ -95,8 +103,8 @@ typedef struct sru_amd_shape {
                               *   SRU_AMD_STATE_INTERVAL steps of each column's walk,
                               *   (max(1, L / SRU_AMD_STATE_INTERVAL), B, D') float; the backward
                               *   call rebuilds the states in between. Refused (BAD_FLAGS) for
-                              *   k = 4 without a skip term, for is_custom together with tanh, and
-                              *   for 16-bit streams with an odd `hidden`. This is the mode the fast
+                              *   k = 4 without a skip term, for is_custom together with tanh, for
+                              *   16-bit streams with an odd `hidden`, and for double streams. This is the mode the fast
                               *   kernels of every shape are built for; with 0 / 1 the 16-bit
                               *   kernels for few columns and the checkpoint backward kernels are
                               *   not available. No counterpart in the reference. */
@@ -107,7 +115,8 @@ typedef struct sru_amd_shape {
                               * is cast). Needs skip_type 1 (otherwise x is not read and the field is
                               * ignored), is_custom 0, activation_type 0, an even `hidden`, and the
                               * state as checkpoints or not at all (BAD_FLAGS otherwise). With dtype
-                              * SRU_AMD_F32 both values mean the same. */
+                              * SRU_AMD_F32 both values mean the same; with SRU_AMD_F64 the field is
+                              * ignored (x is double). */
 } sru_amd_shape;
 
 #define SRU_AMD_X_AS_STREAMS 0
@@ -130,9 +139,9 @@ typedef struct sru_amd_shape {
  *            reference assembles as cat(c[-1, :, :d], c[0, :, d:]) */
 int sru_amd_forward(const sru_amd_shape *shape,
                     const void *u, const void *x, const void *weight_c,
-                    const float *bias, const float *c_init, const float *mask_c,
-                    const uint8_t *mask_pad, const float *scale_x,
-                    void *h, void *c, float *c_last, void *stream);
+                    const void *bias, const void *c_init, const void *mask_c,
+                    const uint8_t *mask_pad, const void *scale_x,
+                    void *h, void *c, void *c_last, void *stream);
 
 /* Bytes of the state buffer `c` that sru_amd_forward fills and sru_amd_backward reads for
  * `shape`, according to shape->state_interval (0 on a bad shape). */
@@ -153,19 +162,19 @@ size_t sru_amd_backward_workspace_bytes(const sru_amd_shape *shape);
  *   grad_last gradient of c_last; NULL = zeros (the usual case: the last state is not part of
  *             the loss)
  *   grad_x    required iff skip_type == 1; already multiplied by scale_x
- *   grad_wc   (2, D') float summed over time and batch, or, when is_custom,
+ *   grad_wc   (2, D') small, summed over time and batch, or, when is_custom,
  *             (L, B, D', 2) in `dtype`
- *   grad_bias (2, D') float summed over time and batch
+ *   grad_bias (2, D') small, summed over time and batch
  *   workspace device scratch of at least sru_amd_backward_workspace_bytes()
  *             bytes, 16-byte aligned; contents before and after are undefined
  * The batch sums are formed in a fixed order: results are bit-reproducible. */
 int sru_amd_backward(const sru_amd_shape *shape,
                      const void *u, const void *x, const void *weight_c,
-                     const float *bias, const float *c_init, const float *mask_c,
-                     const uint8_t *mask_pad, const float *scale_x,
-                     const void *c, const void *grad_h, const float *grad_last,
-                     void *grad_u, void *grad_x, void *grad_wc, float *grad_bias,
-                     float *grad_init, void *workspace, size_t workspace_bytes,
+                     const void *bias, const void *c_init, const void *mask_c,
+                     const uint8_t *mask_pad, const void *scale_x,
+                     const void *c, const void *grad_h, const void *grad_last,
+                     void *grad_u, void *grad_x, void *grad_wc, void *grad_bias,
+                     void *grad_init, void *workspace, size_t workspace_bytes,
                      void *stream);
 
 /* sru_amd_backward without the workspace argument, for callers that cannot allocate device
@@ -174,8 +183,8 @@ int sru_amd_backward(const sru_amd_shape *shape,
  * sru/csrc/sru_cuda_impl.cpp:225-229). The per-column partial sums live in an array built into
  * the library's device code (4 floats per column, 4 MiB, one copy per GPU for the life of the
  * process), so the call allocates nothing and asks for nothing beyond inputs and outputs.
- *   - at most SRU_AMD_STATIC_MAX_COLUMNS columns (B * D'); more returns
- *     SRU_AMD_ERR_STATIC_LIMIT and launches nothing;
+ *   - at most SRU_AMD_STATIC_MAX_COLUMNS columns (B * D'; half as many with SRU_AMD_F64, whose
+ *     partial sums are doubles); more returns SRU_AMD_ERR_STATIC_LIMIT and launches nothing;
  *   - results are bit-identical to sru_amd_backward's (same kernels);
  *   - all calls on one GPU share that GPU's array: two calls that overlap in time on one GPU
  *     (different streams, or two host threads) race; calls on one stream are safe back to back;
@@ -184,11 +193,11 @@ int sru_amd_backward(const sru_amd_shape *shape,
 #define SRU_AMD_STATIC_MAX_COLUMNS 262144
 int sru_amd_backward_static(const sru_amd_shape *shape,
                             const void *u, const void *x, const void *weight_c,
-                            const float *bias, const float *c_init, const float *mask_c,
-                            const uint8_t *mask_pad, const float *scale_x,
-                            const void *c, const void *grad_h, const float *grad_last,
-                            void *grad_u, void *grad_x, void *grad_wc, float *grad_bias,
-                            float *grad_init, void *stream);
+                            const void *bias, const void *c_init, const void *mask_c,
+                            const uint8_t *mask_pad, const void *scale_x,
+                            const void *c, const void *grad_h, const void *grad_last,
+                            void *grad_u, void *grad_x, void *grad_wc, void *grad_bias,
+                            void *grad_init, void *stream);
 
 /* Layer normalisation of the rows of a (rows, cols) matrix, the operation the reference applies to a
  * layer's input before the projection or to its output after the recurrence with

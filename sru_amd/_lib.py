@@ -9,12 +9,12 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsru_amd.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 STATE_INTERVAL = 8   # SRU_AMD_STATE_INTERVAL
 STATIC_MAX_COLUMNS = 262144   # SRU_AMD_STATIC_MAX_COLUMNS
 NORM_MAX_FEATURES = 4096       # SRU_AMD_NORM_MAX_FEATURES
 
-F32, F16, BF16 = 0, 1, 2
+F32, F16, BF16, F64 = 0, 1, 2, 3
 X_AS_STREAMS, X_F32 = 0, 1   # SRU_AMD_X_AS_STREAMS, SRU_AMD_X_F32
 
 

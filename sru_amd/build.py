@@ -9,7 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SOURCES = [os.path.join(HERE, "csrc", n)
            for n in ("sru_amd.hip", "sru_norm.hip", "scan_f32_fwd.hip", "scan_f32_bwd.hip", "scan_f16_fwd.hip",
-                     "scan_f16_bwd.hip", "scan_bf16_fwd.hip", "scan_bf16_bwd.hip")]
+                     "scan_f16_bwd.hip", "scan_bf16_fwd.hip", "scan_bf16_bwd.hip", "scan_f64.hip")]
 OUTPUT = os.path.join(HERE, "libsru_amd.so")
 OBJ_DIR = os.path.join(HERE, "csrc", "build")
 SERVE_FORWARD = os.path.join(HERE, "serve_forward")

@@ -1,10 +1,12 @@
-// Kernel selection for one stream element type T. Included by scan_<type>_fwd.hip and scan_<type>_bwd.hip only.
+// Kernel selection for one stream element type T. Included by scan_<type>_fwd.hip, scan_<type>_bwd.hip and
+// scan_f64.hip only.
 //
 // Fast kernels exist for the three layouts the SRU layer produces without a per-step
 // weight_c: (k=3, skip from x), (k=3, no skip term) and (k=4, skip from U[..., 3]); whether a
 // padding mask is given, whether and how c is stored and the activation are compiled in.
 // Everything else (per-step weight_c; k=4 without a skip term, which the layer never
-// produces) runs the general kernels, one column per lane.
+// produces) runs the general kernels, one column per lane. Double streams run the general
+// kernels for everything, computing in double.
 //
 // Every launcher returns the status of its own hipLaunchKernel call; nothing here reads or
 // clears the runtime's sticky error state, which may hold an error of the embedding program.
@@ -22,6 +24,8 @@ namespace sru_amd {
 // for dword-granular accesses.
 template <typename T> struct Tune { static constexpr int kCols = sizeof(T) == 2 ? 2 : 1; };
 constexpr int kRingDepth = 8;  // ring kernels (reference-style state, general modes)
+// (double streams: a slot is twice as wide, so half the slots keep the ring in registers)
+template <typename T> constexpr int general_ring_depth() { return sizeof(T) == 8 ? kRingDepth / 2 : kRingDepth; }
 // Every large stream is touched exactly once per kernel, so loads and stores are marked
 // non-temporal: measured at the headline shape with cache-cold operands, forward + backward
 // 447 us -> 425 us (float), 230 us -> 214 us (bfloat16).
@@ -167,11 +171,11 @@ inline bool all_aligned_16(std::initializer_list<const void *> ptrs) {
 
 template <typename T, int K, int SKIP>
 hipError_t general_forward(const FwdParams &p, hipStream_t st) {
-    return launch_grouped(forward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, p.ncols, 1, 4, st, p);
+    return launch_grouped(forward_scan<T, K, SKIP, kGeneral | kNt, 1, general_ring_depth<T>()>, p.ncols, 1, 4, st, p);
 }
 template <typename T, int K, int SKIP>
 hipError_t general_backward(const BwdParams &p, hipStream_t st) {
-    return launch_grouped(backward_scan<T, K, SKIP, kGeneral | kNt, 1, kRingDepth>, p.ncols, 1, 4, st, p);
+    return launch_grouped(backward_scan<T, K, SKIP, kGeneral | kNt, 1, general_ring_depth<T>()>, p.ncols, 1, 4, st, p);
 }
 
 // 16-bit streams whose columns cannot be paired (odd d, or a stream pointer that is not aligned to a
@@ -245,17 +249,19 @@ hipError_t custom_backward(const BwdParams &p, hipStream_t st) {
 
 template <typename T>
 hipError_t launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_t st) {
-    if (s.k == 3 ? custom_chunked_ok<T, 3>(s, p.c != nullptr, {p.u}, {p.wc}, {p.x, p.h})
-                 : custom_chunked_ok<T, 4>(s, p.c != nullptr, {p.u}, {p.wc}, {p.x, p.h})) {
-        if (s.k == 4) return custom_forward<T, 4, 2>(p, st);
-        if (s.skip_type == 1) return custom_forward<T, 3, 1>(p, st);
-        return custom_forward<T, 3, 0>(p, st);
-    }
-    const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
-    if (!general) {
-        if (s.k == 4) return pick_forward<T, 4, 2>(s, p, st);
-        if (s.skip_type == 1) return pick_forward<T, 3, 1>(s, p, st);
-        return pick_forward<T, 3, 0>(s, p, st);
+    if constexpr (sizeof(T) != 8) {
+        if (s.k == 3 ? custom_chunked_ok<T, 3>(s, p.c != nullptr, {p.u}, {p.wc}, {p.x, p.h})
+                     : custom_chunked_ok<T, 4>(s, p.c != nullptr, {p.u}, {p.wc}, {p.x, p.h})) {
+            if (s.k == 4) return custom_forward<T, 4, 2>(p, st);
+            if (s.skip_type == 1) return custom_forward<T, 3, 1>(p, st);
+            return custom_forward<T, 3, 0>(p, st);
+        }
+        const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
+        if (!general) {
+            if (s.k == 4) return pick_forward<T, 4, 2>(s, p, st);
+            if (s.skip_type == 1) return pick_forward<T, 3, 1>(s, p, st);
+            return pick_forward<T, 3, 0>(s, p, st);
+        }
     }
     if (s.k == 3 && s.skip_type == 1) return general_forward<T, 3, 1>(p, st);
     if (s.k == 3) return general_forward<T, 3, 0>(p, st);
@@ -265,19 +271,21 @@ hipError_t launch_forward(const sru_amd_shape &s, const FwdParams &p, hipStream_
 
 template <typename T>
 hipError_t launch_backward(const sru_amd_shape &s, const BwdParams &p, hipStream_t st) {
-    if (s.k == 3 ? custom_chunked_ok<T, 3>(s, p.ckpt == nullptr, {p.u, p.gu}, {p.wc, p.gwc_steps}, {p.x, p.gh, p.gx})
-                 : custom_chunked_ok<T, 4>(s, p.ckpt == nullptr, {p.u, p.gu}, {p.wc, p.gwc_steps}, {p.x, p.gh, p.gx})) {
-        if (s.k == 4) return custom_backward<T, 4, 2>(p, st);
-        if (s.skip_type == 1) return custom_backward<T, 3, 1>(p, st);
-        return custom_backward<T, 3, 0>(p, st);
+    if constexpr (sizeof(T) != 8) {
+        if (s.k == 3 ? custom_chunked_ok<T, 3>(s, p.ckpt == nullptr, {p.u, p.gu}, {p.wc, p.gwc_steps}, {p.x, p.gh, p.gx})
+                     : custom_chunked_ok<T, 4>(s, p.ckpt == nullptr, {p.u, p.gu}, {p.wc, p.gwc_steps}, {p.x, p.gh, p.gx})) {
+            if (s.k == 4) return custom_backward<T, 4, 2>(p, st);
+            if (s.skip_type == 1) return custom_backward<T, 3, 1>(p, st);
+            return custom_backward<T, 3, 0>(p, st);
+        }
+        const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
+        if (!general) {
+            if (s.k == 4) return pick_backward<T, 4, 2>(s, p, st);
+            if (s.skip_type == 1) return pick_backward<T, 3, 1>(s, p, st);
+            return pick_backward<T, 3, 0>(s, p, st);
+        }
     }
-    if (s.is_custom && p.ckpt) return hipErrorInvalidValue;   // (refused by the shape and alignment checks before)
-    const bool general = s.is_custom != 0 || (s.skip_type == 0 && s.k == 4);
-    if (!general) {
-        if (s.k == 4) return pick_backward<T, 4, 2>(s, p, st);
-        if (s.skip_type == 1) return pick_backward<T, 3, 1>(s, p, st);
-        return pick_backward<T, 3, 0>(s, p, st);
-    }
+    if (p.ckpt) return hipErrorInvalidValue;   // the general kernels read the state after every step (refused by the shape and alignment checks before)
     if (s.k == 3 && s.skip_type == 1) return general_backward<T, 3, 1>(p, st);
     if (s.k == 3) return general_backward<T, 3, 0>(p, st);
     if (s.skip_type == 2) return general_backward<T, 4, 2>(p, st);

@@ -1,5 +1,6 @@
 // Host-side launchers of the scan kernels, one explicit instantiation per stream element
-// type and pass (scan_f32_fwd.hip, scan_f32_bwd.hip, ... scan_bf16_bwd.hip) so the six compile in parallel.
+// type and pass (scan_f32_fwd.hip, scan_f32_bwd.hip, ... scan_bf16_bwd.hip; scan_f64.hip holds both passes)
+// so that they compile in parallel.
 #pragma once
 
 #include <hip/hip_runtime.h>

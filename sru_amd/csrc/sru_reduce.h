@@ -12,10 +12,12 @@ namespace sru_amd {
 // indices and per quantity; its 16 wavefronts take every 16th batch row each (loads of
 // a wavefront are 256 contiguous bytes), accumulate in double and are combined through
 // LDS in a fixed order, so the result does not depend on scheduling.
+// A: float, or double for double streams (partial sums and results in one type).
 constexpr int kReduceSlices = 16;
 
+template <typename A>
 __global__ void __launch_bounds__(64 * kReduceSlices)
-reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t B, int32_t Dp) {
+reduce_partials(const A *partial, A *grad_wc, A *grad_bias, int64_t B, int32_t Dp) {
     __shared__ double acc[kReduceSlices][64];
     const int lane = threadIdx.x & 63;
     const int slice = threadIdx.x >> 6;
@@ -23,11 +25,11 @@ reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t 
     const int q = blockIdx.y;  // 0 gwc1, 1 gwc2, 2 gbias1, 3 gbias2
     double sum = 0.0;
     if (j < Dp) {
-        const float *src = partial + ((int64_t)q * B) * Dp + j;
+        const A *src = partial + ((int64_t)q * B) * Dp + j;
         int64_t b = slice;
         for (; b + 3 * kReduceSlices < B; b += 4 * kReduceSlices) {  // 4 loads in flight
-            const float v0 = src[b * Dp], v1 = src[(b + kReduceSlices) * Dp];
-            const float v2 = src[(b + 2 * kReduceSlices) * Dp], v3 = src[(b + 3 * kReduceSlices) * Dp];
+            const A v0 = src[b * Dp], v1 = src[(b + kReduceSlices) * Dp];
+            const A v2 = src[(b + 2 * kReduceSlices) * Dp], v3 = src[(b + 3 * kReduceSlices) * Dp];
             sum += (double)v0;
             sum += (double)v1;
             sum += (double)v2;
@@ -41,15 +43,16 @@ reduce_partials(const float *partial, float *grad_wc, float *grad_bias, int64_t 
         double total = acc[0][lane];
 #pragma unroll
         for (int s = 1; s < kReduceSlices; ++s) total += acc[s][lane];
-        float *dst = (q < 2) ? grad_wc : grad_bias;
-        if (dst) dst[(q & 1) * Dp + j] = (float)total;
+        A *dst = (q < 2) ? grad_wc : grad_bias;
+        if (dst) dst[(q & 1) * Dp + j] = (A)total;
     }
 }
 
-inline hipError_t launch_reduce(const float *partial, float *grad_wc, float *grad_bias, int64_t B, int32_t Dp,
+template <typename A>
+inline hipError_t launch_reduce(const A *partial, A *grad_wc, A *grad_bias, int64_t B, int32_t Dp,
                                 hipStream_t st) {
     void *args[] = {&partial, &grad_wc, &grad_bias, &B, &Dp};
-    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_partials), dim3((unsigned)((Dp + 63) / 64), 4),
+    return hipLaunchKernel(reinterpret_cast<const void *>(reduce_partials<A>), dim3((unsigned)((Dp + 63) / 64), 4),
                            dim3(64 * kReduceSlices), args, 0, st);
 }
 

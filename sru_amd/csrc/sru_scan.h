@@ -39,6 +39,12 @@ template <typename T> constexpr int max_waves_per_group(int mode) {
 struct half_bits { uint16_t v; };  // IEEE binary16 storage
 struct bf16_bits { uint16_t v; };  // bfloat16 storage
 
+// Arithmetic type of a stream element type: double streams are computed in double (gates, state,
+// sums and every small tensor; the general kernels only), everything else in float.
+template <typename T> struct Arith { using type = float; };
+template <> struct Arith<double> { using type = double; };
+template <typename T> using arith_t = typename Arith<T>::type;
+
 // ---------------------------------------------------------------- 16-bit conversion
 template <typename T> __device__ __forceinline__ float bits_to_float(uint32_t h);  // h < 65536
 template <> __device__ __forceinline__ float bits_to_float<half_bits>(uint32_t h) {
@@ -101,8 +107,10 @@ template <int W> struct Words<W, false> {  // 6 or 8 dwords: two vectors of 3 or
     }
 };
 
-// storage kind: 0 float, 1 even count of 16-bit elements, 2 odd count of 16-bit elements
-template <typename T, int N> constexpr int group_kind() { return sizeof(T) == 4 ? 0 : (N % 2 == 0 ? 1 : 2); }
+// storage kind: 0 float, 1 even count of 16-bit elements, 2 odd count of 16-bit elements, 3 double
+template <typename T, int N> constexpr int group_kind() {
+    return sizeof(T) == 8 ? 3 : sizeof(T) == 4 ? 0 : (N % 2 == 0 ? 1 : 2);
+}
 
 template <typename T, int N, int KIND = group_kind<T, N>()> struct Group;
 
@@ -150,6 +158,26 @@ struct alignas(2) Group<T, N, 2> {
     }
 };
 
+// doubles: two dwords each (1 to 4 elements: one vector, or two vectors of 3 or 4 dwords)
+template <int N>
+struct Group<double, N, 3> {
+    static constexpr int kWords = 2 * N;
+    Words<2 * N> w;
+    __device__ __forceinline__ double get(int i) const {
+        return __builtin_bit_cast(double, (uint64_t)w.get(2 * i) | ((uint64_t)w.get(2 * i + 1) << 32));
+    }
+    __device__ __forceinline__ static Group make(const double (&v)[N]) {
+        Group g;
+#pragma unroll
+        for (int i = 0; i < N; ++i) {
+            const uint64_t b = __builtin_bit_cast(uint64_t, v[i]);
+            g.w.set(2 * i, (uint32_t)b);
+            g.w.set(2 * i + 1, (uint32_t)(b >> 32));
+        }
+        return g;
+    }
+};
+
 // NT: mark the access non-temporal (streamed once; do not keep the line in the caches);
 // applies to groups that travel as one or two vectors of dwords.
 template <typename T, int N, bool NT = false>
@@ -179,7 +207,7 @@ __device__ __forceinline__ Group<T, N> load_group(const T *p) {
     }
 }
 template <typename T, int N, bool NT = false>
-__device__ __forceinline__ void store_group(T *p, const float (&v)[N]) {
+__device__ __forceinline__ void store_group(T *p, const arith_t<T> (&v)[N]) {
     typedef Group<T, N> G;
     constexpr int W = G::kWords;
     const G g = G::make(v);
@@ -309,9 +337,12 @@ __device__ __forceinline__ float sigmoid_exp2(float t) {
 // add, reciprocal. Float streams keep the sum in its own scale and multiply afterwards: the folded
 // form rounds relative to the terms instead of to their (often much smaller) sum, which doubled the
 // largest gradient error at the headline shape.
+// Double streams: the double-precision exp of the device library (saturates to 0 and 1 through inf
+// like the float forms).
 template <typename T>
-__device__ __forceinline__ float gate(float u, float w, float c, float b) {
-    if constexpr (sizeof(T) == 4) return sigmoid_exp2<T>(kNegLog2e * (u + w * c + b));
+__device__ __forceinline__ arith_t<T> gate(arith_t<T> u, arith_t<T> w, arith_t<T> c, arith_t<T> b) {
+    if constexpr (sizeof(T) == 8) return 1.0 / (1.0 + exp(-(u + w * c + b)));
+    else if constexpr (sizeof(T) == 4) return sigmoid_exp2<T>(kNegLog2e * (u + w * c + b));
     else return sigmoid_exp2<T>(__builtin_fmaf(kNegLog2e * w, c, __builtin_fmaf(kNegLog2e, u, kNegLog2e * b)));
 }
 
@@ -321,8 +352,19 @@ __device__ __forceinline__ float gate(float u, float w, float c, float b) {
 __device__ __forceinline__ float tanh_fast(float v) {
     return 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(2.8853900817779268f * v));
 }
+template <typename T>
+__device__ __forceinline__ arith_t<T> tanh_of(arith_t<T> v) {
+    if constexpr (sizeof(T) == 8) return tanh(v);
+    else return tanh_fast(v);
+}
 
 // ---------------------------------------------------------------- kernel parameters
+// The small tensors (bias, initial state, masks, scale, last state, partial sums) are typed for the
+// float kernels; with double streams they hold doubles and the general kernels read them through
+// as_arith<double>().
+template <typename A> __device__ __forceinline__ const A *as_arith(const float *q) { return reinterpret_cast<const A *>(q); }
+template <typename A> __device__ __forceinline__ A *as_arith(float *q) { return reinterpret_cast<A *>(q); }
+
 struct FwdParams {
     const void *u, *x, *wc;
     const float *bias, *c0, *mask_c;
@@ -404,23 +446,27 @@ constexpr int kCkptInterval = 8;
 // that lives over the whole walk: the running sums of the weight_c / bias gradients have
 // L terms per column, and plain float accumulation of that many terms was the largest single
 // contribution to their error. Four instructions per chunk and sum, not per cell.
-struct CompensatedSum {
-    float sum = 0.f, comp = 0.f;
-    __device__ __forceinline__ void add(float part) {
-        const float y = part - comp;
-        const float t = sum + y;
+template <typename A>
+struct CompensatedSumOf {
+    A sum = 0, comp = 0;
+    __device__ __forceinline__ void add(A part) {
+        const A y = part - comp;
+        const A t = sum + y;
         comp = (t - sum) - y;
         sum = t;
     }
-    __device__ __forceinline__ float value() const { return sum - comp; }
+    __device__ __forceinline__ A value() const { return sum - comp; }
 };
+using CompensatedSum = CompensatedSumOf<float>;
 
 // ================================================================= forward scan
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
 // U[..., 3]. COLS: columns per lane (2 needs an even d). P: ring depth.
 template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock * 4) forward_scan(const FwdParams p) {
+    using A = arith_t<T>;
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
+    static_assert(sizeof(T) != 8 || (GENERAL && COLS == 1), "double streams: the general kernels, one column per lane");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     static_assert((MODE & (kCkpt | kPair | kUniform)) == 0, "those exist in the chunked kernels only");
     const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * COLS;  // lane's first column
@@ -435,17 +481,17 @@ __global__ void __launch_bounds__(kBlock * 4) forward_scan(const FwdParams p) {
     const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
     const bool keep_c = GENERAL ? (p.c != nullptr) : ((MODE & kKeepC) != 0);
 
-    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], cur[COLS];
+    A wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], cur[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        wc1[c] = custom ? 0.f : static_cast<const float *>(p.wc)[j + c];
-        wc2[c] = custom ? 0.f : static_cast<const float *>(p.wc)[Dp + j + c];
-        b1[c] = p.bias[j + c];
-        b2[c] = p.bias[Dp + j + c];
-        m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
-        cur[c] = p.c0 ? p.c0[col + c] : 0.0f;   // no initial state given: zeros
+        wc1[c] = custom ? A(0) : static_cast<const A *>(p.wc)[j + c];
+        wc2[c] = custom ? A(0) : static_cast<const A *>(p.wc)[Dp + j + c];
+        b1[c] = as_arith<A>(p.bias)[j + c];
+        b2[c] = as_arith<A>(p.bias)[Dp + j + c];
+        m[c] = p.mask_c ? as_arith<A>(p.mask_c)[col + c] : A(1);
+        cur[c] = p.c0 ? as_arith<A>(p.c0)[col + c] : A(0);   // no initial state given: zeros
     }
-    const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
+    const A sx = (SKIP == 1 && p.scale_x) ? *as_arith<A>(p.scale_x) : A(1);
 
     const int64_t L = p.L;
     const int64_t e0 = (flip ? (L - 1) : 0) * p.ncols + col;  // element of the first walk step
@@ -485,25 +531,25 @@ __global__ void __launch_bounds__(kBlock * 4) forward_scan(const FwdParams p) {
 
     auto consume = [&](const Slot &s) {
         const bool padded = s.pad != 0;
-        float hv[COLS], cv[COLS];
+        A hv[COLS], cv[COLS];
 #pragma unroll
         for (int c = 0; c < COLS; ++c) {
-            const float u0 = s.u.get(c * K), u1 = s.u.get(c * K + 1), u2 = s.u.get(c * K + 2);
-            const float w1 = custom ? s.w.get(2 * c) : wc1[c];
-            const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
-            const float g1 = gate<T>(u1, w1, cur[c], b1[c]);
-            const float g2 = gate<T>(u2, w2, cur[c], b2[c]);
-            const float cn = (cur[c] - u0) * g1 + u0;
-            const float val = use_tanh ? tanh_fast(cn) : cn;
-            float out;
+            const A u0 = s.u.get(c * K), u1 = s.u.get(c * K + 1), u2 = s.u.get(c * K + 2);
+            const A w1 = custom ? s.w.get(2 * c) : wc1[c];
+            const A w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
+            const A g1 = gate<T>(u1, w1, cur[c], b1[c]);
+            const A g2 = gate<T>(u2, w2, cur[c], b2[c]);
+            const A cn = (cur[c] - u0) * g1 + u0;
+            const A val = use_tanh ? tanh_of<T>(cn) : cn;
+            A out;
             if (SKIP != 0) {
-                const float xv = (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
+                const A xv = (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
                 out = (val - xv) * m[c] * g2 + xv;
             } else {
                 out = val * m[c] * g2;
             }
             cur[c] = padded ? cur[c] : cn;   // a padded step keeps the state ...
-            hv[c] = padded ? 0.0f : out;     // ... and emits zero
+            hv[c] = padded ? A(0) : out;     // ... and emits zero
             cv[c] = cur[c];
         }
         store_group<T, COLS, NTS>(hp, hv);
@@ -540,7 +586,7 @@ __global__ void __launch_bounds__(kBlock * 4) forward_scan(const FwdParams p) {
         }
     }
 #pragma unroll
-    for (int c = 0; c < COLS; ++c) p.c_last[col + c] = cur[c];
+    for (int c = 0; c < COLS; ++c) as_arith<A>(p.c_last)[col + c] = cur[c];
 }
 
 // Window of a wavefront's walk outside of which every step is padded, for wavefronts whose lanes
@@ -776,7 +822,9 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) forward
 // reduce_partials() then adds them over the batch in a fixed order.
 template <typename T, int K, int SKIP, int MODE, int COLS, int P>
 __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
+    using A = arith_t<T>;
     constexpr bool GENERAL = (MODE & kGeneral) != 0;
+    static_assert(sizeof(T) != 8 || (GENERAL && COLS == 1), "double streams: the general kernels, one column per lane");
     constexpr bool NTL = (MODE & kNtLoad) != 0, NTS = (MODE & kNtStore) != 0;
     const int64_t col = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * COLS;
     if (col >= p.ncols) return;
@@ -789,10 +837,10 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
     const bool use_tanh = GENERAL ? (p.act != 0) : ((MODE & kTanh) != 0);
     const bool has_pad = GENERAL ? (p.pad != nullptr) : ((MODE & kHasPad) != 0);
 
-    float wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
-    float cur[COLS];  // d loss / d state
-    float gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];  // sums of the current ring round
-    CompensatedSum sw1[COLS], sw2[COLS], sb1[COLS], sb2[COLS];  // sums over the whole walk
+    A wc1[COLS], wc2[COLS], b1[COLS], b2[COLS], m[COLS], c_init[COLS];
+    A cur[COLS];  // d loss / d state
+    A gw1[COLS], gw2[COLS], gb1[COLS], gb2[COLS];  // sums of the current ring round
+    CompensatedSumOf<A> sw1[COLS], sw2[COLS], sb1[COLS], sb2[COLS];  // sums over the whole walk
     auto fold_round = [&]() {
 #pragma unroll
         for (int c = 0; c < COLS; ++c) {
@@ -800,21 +848,21 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
             sw2[c].add(gw2[c]);
             sb1[c].add(gb1[c]);
             sb2[c].add(gb2[c]);
-            gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
+            gw1[c] = gw2[c] = gb1[c] = gb2[c] = A(0);
         }
     };
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        wc1[c] = custom ? 0.f : static_cast<const float *>(p.wc)[j + c];
-        wc2[c] = custom ? 0.f : static_cast<const float *>(p.wc)[Dp + j + c];
-        b1[c] = p.bias[j + c];
-        b2[c] = p.bias[Dp + j + c];
-        m[c] = p.mask_c ? p.mask_c[col + c] : 1.0f;
-        c_init[c] = p.c0 ? p.c0[col + c] : 0.0f;          // no initial state given: zeros
-        cur[c] = p.glast ? p.glast[col + c] : 0.0f;      // no gradient of the last state given: zeros
-        gw1[c] = gw2[c] = gb1[c] = gb2[c] = 0.f;
+        wc1[c] = custom ? A(0) : static_cast<const A *>(p.wc)[j + c];
+        wc2[c] = custom ? A(0) : static_cast<const A *>(p.wc)[Dp + j + c];
+        b1[c] = as_arith<A>(p.bias)[j + c];
+        b2[c] = as_arith<A>(p.bias)[Dp + j + c];
+        m[c] = p.mask_c ? as_arith<A>(p.mask_c)[col + c] : A(1);
+        c_init[c] = p.c0 ? as_arith<A>(p.c0)[col + c] : A(0);          // no initial state given: zeros
+        cur[c] = p.glast ? as_arith<A>(p.glast)[col + c] : A(0);      // no gradient of the last state given: zeros
+        gw1[c] = gw2[c] = gb1[c] = gb2[c] = A(0);
     }
-    const float sx = (SKIP == 1 && p.scale_x) ? *p.scale_x : 1.0f;
+    const A sx = (SKIP == 1 && p.scale_x) ? *as_arith<A>(p.scale_x) : A(1);
 
     const int64_t L = p.L;
     // The backward walk starts where the forward walk ended.
@@ -832,7 +880,7 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
     T *gxp = (SKIP == 1) ? static_cast<T *>(p.gx) + e0 : nullptr;
     T *gvp = custom ? static_cast<T *>(p.gwc_steps) + e0 * 2 : nullptr;
 
-    float cv[COLS];  // state after the step being visited
+    A cv[COLS];  // state after the step being visited
     {
         const Group<T, COLS> g = load_group<T, COLS>(static_cast<const T *>(p.c) + e0);
 #pragma unroll
@@ -875,37 +923,37 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
 
     auto consume = [&](const Slot &s) {
         const bool padded = s.pad != 0;
-        float gu[COLS * K], gx[COLS], gv[COLS * 2];
+        A gu[COLS * K], gx[COLS], gv[COLS * 2];
 #pragma unroll
         for (int c = 0; c < COLS; ++c) {
-            const float w1 = custom ? s.w.get(2 * c) : wc1[c];
-            const float w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
-            const float cp = s.first ? c_init[c] : s.cprev.get(c);
-            const float u0 = s.u.get(c * K);
-            const float g1 = gate<T>(s.u.get(c * K + 1), w1, cp, b1[c]);
-            const float g2 = gate<T>(s.u.get(c * K + 2), w2, cp, b2[c]);
-            const float val = use_tanh ? tanh_fast(cv[c]) : cv[c];
-            const float dact = use_tanh ? (1.0f - val * val) : 1.0f;
-            const float xv = (SKIP == 0) ? 0.0f : (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
-            const float gh = s.gh.get(c);
+            const A w1 = custom ? s.w.get(2 * c) : wc1[c];
+            const A w2 = custom ? s.w.get(2 * c + 1) : wc2[c];
+            const A cp = s.first ? c_init[c] : s.cprev.get(c);
+            const A u0 = s.u.get(c * K);
+            const A g1 = gate<T>(s.u.get(c * K + 1), w1, cp, b1[c]);
+            const A g2 = gate<T>(s.u.get(c * K + 2), w2, cp, b2[c]);
+            const A val = use_tanh ? tanh_of<T>(cv[c]) : cv[c];
+            const A dact = use_tanh ? (A(1) - val * val) : A(1);
+            const A xv = (SKIP == 0) ? A(0) : (SKIP == 1) ? s.x.get(c) * sx : s.u.get(c * K + K - 1);
+            const A gh = s.gh.get(c);
 
-            const float gg2 = gh * (val - xv) * m[c] * (g2 * (1.0f - g2));
-            const float gc = gh * m[c] * (g2 * dact) + cur[c];
-            const float gg1 = gc * (cp - u0) * (g1 * (1.0f - g1));
-            const float gskip = gh * (1.0f - g2 * m[c]);
-            const float ncur = gc * g1 + gg1 * w1 + gg2 * w2;
+            const A gg2 = gh * (val - xv) * m[c] * (g2 * (A(1) - g2));
+            const A gc = gh * m[c] * (g2 * dact) + cur[c];
+            const A gg1 = gc * (cp - u0) * (g1 * (A(1) - g1));
+            const A gskip = gh * (A(1) - g2 * m[c]);
+            const A ncur = gc * g1 + gg1 * w1 + gg2 * w2;
 
-            gu[c * K] = padded ? 0.0f : gc * (1.0f - g1);
-            gu[c * K + 1] = padded ? 0.0f : gg1;
-            gu[c * K + 2] = padded ? 0.0f : gg2;
-            if (K == 4) gu[c * K + K - 1] = (padded || SKIP != 2) ? 0.0f : gskip;
-            gx[c] = padded ? 0.0f : gskip * sx;
-            gv[2 * c] = padded ? 0.0f : gg1 * cp;
-            gv[2 * c + 1] = padded ? 0.0f : gg2 * cp;
-            gb1[c] += padded ? 0.0f : gg1;
-            gw1[c] += padded ? 0.0f : gg1 * cp;
-            gb2[c] += padded ? 0.0f : gg2;
-            gw2[c] += padded ? 0.0f : gg2 * cp;
+            gu[c * K] = padded ? A(0) : gc * (A(1) - g1);
+            gu[c * K + 1] = padded ? A(0) : gg1;
+            gu[c * K + 2] = padded ? A(0) : gg2;
+            if (K == 4) gu[c * K + K - 1] = (padded || SKIP != 2) ? A(0) : gskip;
+            gx[c] = padded ? A(0) : gskip * sx;
+            gv[2 * c] = padded ? A(0) : gg1 * cp;
+            gv[2 * c + 1] = padded ? A(0) : gg2 * cp;
+            gb1[c] += padded ? A(0) : gg1;
+            gw1[c] += padded ? A(0) : gg1 * cp;
+            gb2[c] += padded ? A(0) : gg2;
+            gw2[c] += padded ? A(0) : gg2 * cp;
             cur[c] = padded ? cur[c] : ncur;
             cv[c] = cp;  // the state before this step is the state after the next one visited
         }
@@ -949,11 +997,11 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
 
 #pragma unroll
     for (int c = 0; c < COLS; ++c) {
-        p.ginit[col + c] = cur[c];
-        p.partial[col + c] = sw1[c].value();
-        p.partial[p.ncols + col + c] = sw2[c].value();
-        p.partial[2 * p.ncols + col + c] = sb1[c].value();
-        p.partial[3 * p.ncols + col + c] = sb2[c].value();
+        as_arith<A>(p.ginit)[col + c] = cur[c];
+        as_arith<A>(p.partial)[col + c] = sw1[c].value();
+        as_arith<A>(p.partial)[p.ncols + col + c] = sw2[c].value();
+        as_arith<A>(p.partial)[2 * p.ncols + col + c] = sb1[c].value();
+        as_arith<A>(p.partial)[3 * p.ncols + col + c] = sb2[c].value();
     }
 }
 

@@ -20,7 +20,9 @@ The large streams (U, x, h, c and their gradients) are consumed in the dtype of
 beside a 16-bit U (the layer's input under autocast, which the reference keeps in
 float32 too, sru/ops.py:121) is read as it is, and grad_x comes back in float32,
 wherever the kernels take it (plain layer: vector weight_c, identity activation, even
-d); elsewhere x is rounded to u's dtype first. A float64 U is computed in float32.
+d); elsewhere x is rounded to u's dtype first. A float64 U runs the double kernels:
+streams, small tensors, state and arithmetic in double, as the reference's kernels
+dispatched for double do (sru/csrc/sru_cuda_kernel.cu:845).
 """
 from typing import Optional, Tuple
 
@@ -33,7 +35,7 @@ from torch.autograd import Function
 
 from . import _lib
 
-_DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+_DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16, torch.float64: _lib.F64}
 
 
 def _ptr(t: Optional[Tensor]):
@@ -77,10 +79,12 @@ def _aligned(t: Tensor, nbytes: int) -> Tensor:
     return t
 
 
-def _f32(t: Optional[Tensor]) -> Optional[Tensor]:
+def _small(t: Optional[Tensor], dtype: torch.dtype) -> Optional[Tensor]:
+    """A small tensor (weight_c vector, bias, initial state, mask, scale, last-state gradient) as the
+    kernels read it: float32, or float64 beside double streams."""
     if t is None:
         return None
-    return _aligned(t if t.dtype == torch.float32 else t.float(), 4)
+    return _aligned(t if t.dtype == dtype else t.to(dtype), 8)
 
 
 class _Problem:
@@ -90,7 +94,7 @@ class _Problem:
     def __init__(self, dtype, x_dim, length, batch, u_numel, u_last, is_custom, d_out,
                  bidirectional, has_skip_term, activation_type, checkpoint_state, x_is_float, state_kept):
         if dtype not in _DTYPES:
-            raise ValueError(f"U must be float32, float16 or bfloat16, not {dtype}")
+            raise ValueError(f"U must be float32, float64, float16 or bfloat16, not {dtype}")
         if x_dim not in (2, 3):
             raise ValueError("x must be 2 or 3 dimensional")
         self.batch = batch
@@ -106,16 +110,19 @@ class _Problem:
         self.skip_type = 0 if not has_skip_term else (1 if self.k == 3 else 2)
         self.activation_type = activation_type
         self.dtype = dtype
+        self.small_dtype = torch.float64 if dtype == torch.float64 else torch.float32
         self.squeeze = x_dim == 2
         # Between forward and backward keep float checkpoints of the state instead of the
         # state after every step wherever the kernels support it (with four streams, a skip
         # term): the backward kernel rebuilds what lies in between.
-        # 16-bit streams need an even d for that; a per-step weight_c must not come with tanh.
-        ok = (dtype == torch.float32 or d_out % 2 == 0) and not (self.is_custom and activation_type != 0)
+        # 16-bit streams need an even d for that; a per-step weight_c must not come with tanh;
+        # double streams run the general kernels, which read the state after every step.
+        ok = (dtype == torch.float32 or d_out % 2 == 0) and not (self.is_custom and activation_type != 0) \
+            and dtype != torch.float64
         self.checkpointed = bool(checkpoint_state and ok and not (self.skip_type == 0 and self.k == 4))
         # A float32 x beside 16-bit streams (the layer's input under autocast) is read as it is by
         # the chunked kernels of the plain layer; everywhere else x is rounded to the stream dtype.
-        self.x_float = bool(x_is_float and dtype != torch.float32 and self.skip_type == 1 and not self.is_custom
+        self.x_float = bool(x_is_float and dtype in (torch.float16, torch.bfloat16) and self.skip_type == 1 and not self.is_custom
                             and activation_type == 0 and d_out % 2 == 0 and (self.checkpointed or not state_kept))
         self.x_dtype = torch.float32 if self.x_float else dtype
         self.shape = _lib.Shape(self.length, self.batch, self.d, self.dirs, self.k,
@@ -127,10 +134,6 @@ class _Problem:
         self.state_rows = lib.sru_amd_state_bytes(ctypes.byref(self.shape)) // (4 * self.batch * self.Dp) \
             if self.checkpointed else self.length
         self.workspace_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(self.shape))
-
-    def group_bytes(self):
-        es = 4 if self.dtype == torch.float32 else 2
-        return es * (4 if self.k == 4 else 1)
 
 
 _problem_cached = functools.lru_cache(maxsize=256)(_Problem)
@@ -162,19 +165,19 @@ def _prepare_inputs(pb: _Problem, u, x, weight_c, bias, init, scale_x, mask_c, m
         if wc_.numel() != pb.length * pb.batch * pb.Dp * 2:
             raise ValueError("per-step weight_c must have length*batch*output_size*2 elements")
     else:
-        wc_ = _f32(weight_c)
+        wc_ = _small(weight_c, pb.small_dtype)
         if wc_.numel() != 2 * pb.Dp:
             raise ValueError("weight_c must have 2*output_size elements")
-    bias_ = _f32(bias)
-    init_ = _f32(init)         # None: the kernels start from zeros
+    bias_ = _small(bias, pb.small_dtype)
+    init_ = _small(init, pb.small_dtype)         # None: the kernels start from zeros
     if bias_.numel() != 2 * pb.Dp or (init_ is not None and init_.numel() != pb.batch * pb.Dp):
         raise ValueError("bias must have 2*output_size and init batch*output_size elements")
-    mask_c_ = _f32(mask_c)
+    mask_c_ = _small(mask_c, pb.small_dtype)
     if mask_c_ is not None and mask_c_.numel() != pb.batch * pb.Dp:
         raise ValueError("mask_c must have batch*output_size elements")
     scale_ = None
     if scale_x is not None and pb.skip_type == 1:
-        scale_ = _f32(scale_x.reshape(-1)[:1])
+        scale_ = _small(scale_x.reshape(-1)[:1], pb.small_dtype)
     pad_ = None
     if mask_pad is not None:
         pad_ = mask_pad.contiguous()
@@ -194,7 +197,7 @@ def _run_forward(pb, u_, x_, wc_, bias_, init_, scale_, mask_c_, pad_, keep_c: b
         c = torch.empty(pb.state_rows, pb.batch, pb.Dp, dtype=torch.float32, device=dev)
     elif keep_c:
         c = torch.empty(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
-    c_last = torch.empty(pb.batch, pb.Dp, dtype=torch.float32, device=dev)
+    c_last = torch.empty(pb.batch, pb.Dp, dtype=pb.small_dtype, device=dev)
     with _on_device(dev) as stream:
         rc = lib.sru_amd_forward(ctypes.byref(pb.shape), _ptr(u_), _ptr(x_), _ptr(wc_), _ptr(bias_),
                                  _ptr(init_), _ptr(mask_c_), _ptr(pad_), _ptr(scale_), _ptr(h),
@@ -204,10 +207,9 @@ def _run_forward(pb, u_, x_, wc_, bias_, init_, scale_, mask_c_, pad_, keep_c: b
 
 
 def _kernel_dtype(u: Tensor) -> torch.dtype:
-    """Stream dtype the kernels run in for a U of this dtype: float16 and bfloat16 as they are,
-    everything else float32 (float64 included: the reference's training entry casts it to float32
-    as well, sru/ops.py:116-127)."""
-    return u.dtype if u.dtype in (torch.float16, torch.bfloat16) else torch.float32
+    """Stream dtype the kernels run in for a U of this dtype: the four the kernels exist for as
+    they are, anything else float32."""
+    return u.dtype if u.dtype in _DTYPES else torch.float32
 
 
 def elementwise_recurrence_forward(
@@ -220,7 +222,6 @@ def elementwise_recurrence_forward(
 
     `keep_c=False` (no counterpart in the reference) skips storing the per-step
     state and returns None for it: the inference variant. `init=None` stands for zeros.
-    A float64 U is computed in float32 and the results are cast back.
     """
     out_dtype = u.dtype
     if u.dtype != _kernel_dtype(u):
@@ -228,7 +229,7 @@ def elementwise_recurrence_forward(
     pb = _problem(u, x, weight_c, d_out, bidirectional, has_skip_term, activation_type, state_kept=keep_c)
     prepared = _prepare_inputs(pb, u, x, weight_c, bias, init, scale_x, mask_c, mask_pad)
     h, c, c_last = _run_forward(pb, *prepared, keep_c=keep_c)
-    last_hidden = c_last if out_dtype == torch.float32 else c_last.to(out_dtype)
+    last_hidden = c_last if out_dtype == c_last.dtype else c_last.to(out_dtype)
     if out_dtype != pb.dtype:
         h = h.to(out_dtype)
         c = c.to(out_dtype) if c is not None else None
@@ -241,9 +242,9 @@ def elementwise_recurrence_forward(
 class ElementwiseRecurrence(Function):
     """Drop-in for sru/cuda_functional.py:156-261.
 
-    Beyond the reference's argument list: `init` may be None (zeros, and no gradient for it). A
-    float64 U (which the reference's kernels compute in double) is computed in float32 here; outputs
-    and gradients come back in the dtypes of the inputs."""
+    Beyond the reference's argument list: `init` may be None (zeros, and no gradient for it).
+    Outputs come back in U's dtype and gradients in the dtypes of the inputs; a float64 U is
+    computed in double, so torch.autograd.gradcheck applies to this Function as it is."""
 
     @staticmethod
     def forward(ctx, u, x, weight_c, bias, init, activation_type, d_out, bidirectional,
@@ -263,7 +264,7 @@ class ElementwiseRecurrence(Function):
         ctx.in_shapes = (u.shape, x.shape, weight_c.shape, bias.shape, None if init is None else init.shape)
         ctx.save_for_backward(*[t for t in prepared if t is not None], c)
         ctx.present = [t is not None for t in prepared]
-        last_hidden = c_last if u_dtype == torch.float32 else c_last.to(u_dtype)
+        last_hidden = c_last if u_dtype == c_last.dtype else c_last.to(u_dtype)
         if u_dtype != pb.dtype:
             h = h.to(u_dtype)
         if pb.squeeze:
@@ -282,13 +283,13 @@ class ElementwiseRecurrence(Function):
             gh = torch.zeros(pb.length, pb.batch, pb.Dp, dtype=pb.dtype, device=dev)
         else:
             gh = _aligned(grad_h if grad_h.dtype == pb.dtype else grad_h.to(pb.dtype), 4)
-        gl = _f32(grad_last)   # None: the kernels start from a zero state gradient
+        gl = _small(grad_last, pb.small_dtype)   # None: the kernels start from a zero state gradient
         grad_u = torch.empty_like(u_)
         grad_x = torch.empty_like(x_) if pb.skip_type == 1 else None
         grad_wc = torch.empty_like(wc_) if pb.is_custom else \
-            torch.empty(2 * pb.Dp, dtype=torch.float32, device=dev)
+            torch.empty(2 * pb.Dp, dtype=pb.small_dtype, device=dev)
         # grad_bias (2, D') and grad_init (B, D') share one allocation
-        small = torch.empty((2 + pb.batch) * pb.Dp, dtype=torch.float32, device=dev)
+        small = torch.empty((2 + pb.batch) * pb.Dp, dtype=pb.small_dtype, device=dev)
         grad_bias, grad_init = small[:2 * pb.Dp], small[2 * pb.Dp:]
         ws_bytes = pb.workspace_bytes
         workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)

@@ -17,7 +17,10 @@ from torch import Tensor
 from torch.autograd import Function
 
 from . import _lib
-from .functional import _DTYPES, _aligned, _f32, _on_device, _ptr
+from .functional import _aligned, _on_device, _ptr, _small
+
+# element types the layer-norm kernels read and write (no double rows)
+_DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
 
 
 def supported(x: Tensor) -> bool:
@@ -30,7 +33,7 @@ class LayerNormFunction(Function):
     def forward(ctx, x, weight, bias, eps, out_dtype):
         D = x.size(-1)
         x_ = _aligned(x, 16)
-        w_, b_ = _aligned(_f32(weight), 16), _aligned(_f32(bias), 16)
+        w_, b_ = _aligned(_small(weight, torch.float32), 16), _aligned(_small(bias, torch.float32), 16)
         rows = x_.numel() // D
         y = torch.empty(x_.shape, dtype=out_dtype, device=x.device)
         mean = torch.empty(rows, dtype=torch.float32, device=x.device)
@@ -75,7 +78,7 @@ def layer_norm(x: Tensor, weight: Tensor, bias: Tensor, eps: float = 1e-5,
     A tensor the kernels do not take (see `supported`) goes through torch's own layer_norm, once
     per feature count with a warning; `strict=True` raises instead."""
     out_dtype = out_dtype or x.dtype
-    if out_dtype not in _DTYPES:
+    if out_dtype not in _DTYPES and x.dtype in _DTYPES:
         raise ValueError(f"out_dtype must be float32, float16 or bfloat16, not {out_dtype}")
     if not supported(x):
         why = (f"sru_amd.norm.layer_norm: no kernel for a {x.dtype} {'device' if x.is_cuda else 'CPU'} tensor with "
@@ -86,6 +89,7 @@ def layer_norm(x: Tensor, weight: Tensor, bias: Tensor, eps: float = 1e-5,
         if key not in _warned_widths:
             _warned_widths.add(key)
             warnings.warn(why + "; using torch.nn.functional.layer_norm")
-        y = torch.nn.functional.layer_norm(x.float(), (x.size(-1),), weight.float(), bias.float(), eps)
+        wide = torch.float64 if x.dtype == torch.float64 else torch.float32
+        y = torch.nn.functional.layer_norm(x.to(wide), (x.size(-1),), weight.to(wide), bias.to(wide), eps)
         return y.to(out_dtype)
     return LayerNormFunction.apply(x, weight, bias, eps, out_dtype)

@@ -11,7 +11,8 @@ whatever the stream dtype, so the `.float()` copies of U and x are not needed:
 with `native_16bit=True` (default) a float16 / bfloat16 U is read as is and h
 comes back in that dtype; `native_16bit=False` reproduces the reference's
 float32 casts (h is then float32, as in the reference). Any other dtype (float64)
-is cast to float32 as in the reference, and h is float32.
+is cast to float32 as in the reference, and h is float32; double kernels exist
+behind `ElementwiseRecurrence.apply` called directly, as in the reference.
 
 `c_init` may be None (no counterpart in the reference): the kernels then start from zeros
 without a zero tensor being allocated and filled.

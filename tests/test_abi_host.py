@@ -43,7 +43,7 @@ FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: validation fails first
     (dict(length=1 << 60), 2), (dict(dirs=3), 3), (dict(k=5), 3), (dict(k=2), 3),
     (dict(activation_type=2), 3), (dict(skip_type=3), 3), (dict(skip_type=1, k=4), 3),
     (dict(skip_type=2, k=3), 3), (dict(is_custom=2), 3), (dict(dtype=7), 4),
-    (dict(state_interval=4), 3),
+    (dict(state_interval=4), 3), (dict(state_interval=8, dtype=3), 3),   # double streams: no checkpoints
     (dict(state_interval=8, is_custom=1, activation_type=1), 3), (dict(state_interval=8, skip_type=0, k=4), 3),
     (dict(state_interval=8, dtype=2, hidden=7), 3), (dict(state_interval=8, dtype=1, hidden=1), 3),
     # a float x beside 16-bit streams: plain layer only, even hidden; with float streams the field changes nothing
@@ -82,6 +82,12 @@ def test_null_and_misaligned_pointers_and_workspace():
     assert lib.sru_amd_state_bytes(ctypes.byref(_shape(dtype=2))) == 4 * 2 * 16 * 2
     assert lib.sru_amd_state_bytes(ctypes.byref(_shape(state_interval=8))) == 1 * 2 * 16 * 4
     assert lib.sru_amd_state_bytes(ctypes.byref(_shape(length=33, state_interval=8, dtype=1))) == 4 * 2 * 16 * 4
+    # double streams: the state after every step in double, and double partial sums
+    assert lib.sru_amd_state_bytes(ctypes.byref(_shape(dtype=3))) == 4 * 2 * 16 * 8
+    assert lib.sru_amd_backward_workspace_bytes(ctypes.byref(_shape(dtype=3))) == 4 * 8 * 2 * 16
+    bad = list(args)
+    bad[3] = ctypes.c_void_p(0x1004)            # with double streams the small tensors are doubles too
+    assert lib.sru_amd_forward(ctypes.byref(_shape(dtype=3)), *bad, None) == 5
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 16), None, need, None) == 6
     assert lib.sru_amd_backward(ctypes.byref(s), *([FAKE] * 17), need - 1, None) == 6
     # u, x, weight_c, bias, c, grad_h, grad_u, grad_x, grad_wc, grad_bias, grad_init
@@ -108,6 +114,8 @@ def test_static_backward_checks_sizes_before_anything_else():
     lib = _lib.load()
     wide = _shape(batch=_lib.STATIC_MAX_COLUMNS // 16 + 1)
     assert lib.sru_amd_backward_static(ctypes.byref(wide), *([FAKE] * 16), None) == 8
+    half = _shape(batch=_lib.STATIC_MAX_COLUMNS // 32 + 1, dtype=3)   # double partial sums: half the columns
+    assert lib.sru_amd_backward_static(ctypes.byref(half), *([FAKE] * 16), None) == 8
     assert lib.sru_amd_backward_static(ctypes.byref(_shape(k=5)), *([FAKE] * 16), None) == 3
     assert lib.sru_amd_backward_static(None, *([FAKE] * 16), None) == 1
 
@@ -119,7 +127,7 @@ def test_layer_norm_entry_points_validate_before_launching():
         rows, cols, x, dx, FAKE, FAKE, ctypes.c_float(1e-5), FAKE, dy, FAKE, FAKE, None)
     assert fwd(0, 64) == 2 and fwd(4, 0) == 2 and fwd(4, 12) == 2          # cols must be a multiple of 8
     assert fwd(4, _lib.NORM_MAX_FEATURES + 8) == 2
-    assert fwd(4, 64, dx=9) == 4 and fwd(4, 64, dy=5) == 4
+    assert fwd(4, 64, dx=9) == 4 and fwd(4, 64, dy=5) == 4 and fwd(4, 64, dx=3) == 4   # no double rows
     assert fwd(4, 64, x=None) == 1
     assert fwd(4, 64, x=ctypes.c_void_p(0x1004)) == 5
     need = lib.sru_amd_layer_norm_backward_workspace_bytes(4, 64)

@@ -88,17 +88,17 @@ def test_amp_style_bf16_streams_against_fp32_run():
         assert float((a - b).detach().abs().max()) <= 2e-2 * max(1.0, float(b.detach().abs().max()))
 
 
-def test_float64_inputs_are_computed_in_float32_and_come_back_as_given():
-    # the reference's training entry casts float64 to float32 and returns float32 (sru/ops.py:116-127);
-    # its autograd Function, called directly, keeps the dtype of U (its kernels exist for double,
-    # sru/csrc/sru_cuda_kernel.cu:845). Here both compute in float32.
+def test_float64_function_runs_in_double_and_training_entry_casts_to_float32():
+    # the reference's autograd Function, called directly, keeps the dtype of U and its kernels exist
+    # for double (sru/csrc/sru_cuda_kernel.cu:845); its training entry casts float64 to float32 and
+    # returns float32 (sru/ops.py:116-127). Same here.
     from sru_amd import ElementwiseRecurrence, elementwise_recurrence_gpu
-    c = Case(L=14, B=3, d=64, dirs=2, seed=44, pad="right", scale=1.7, mask_c=True).f32()
+    c = Case(L=14, B=3, d=64, dirs=2, seed=44, pad="right", scale=1.7, mask_c=True)
     h64, last64, g64 = _apply(ElementwiseRecurrence.apply, c, "cuda:0", torch.float64)
     h_ref, last_ref, g_ref = _apply(st.recurrence, c, "cpu", torch.float64)
-    assert np.abs(h64 - h_ref).max() <= 1e-5 and np.abs(last64 - last_ref).max() <= 1e-5
+    assert np.abs(h64 - h_ref).max() <= 1e-12 and np.abs(last64 - last_ref).max() <= 1e-12
     for a, b in zip(g64, g_ref):
-        assert a is not None and np.abs(a - b).max() <= 1e-5 * max(1.0, np.abs(b).max())
+        assert a is not None and np.abs(a - b).max() <= 1e-12 * max(1.0, np.abs(b).max())
     dev = "cuda:0"
     t = lambda a: torch.tensor(a, dtype=torch.float64, device=dev, requires_grad=True)
     u, x, wc, bias, c0 = t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0)
@@ -111,6 +111,29 @@ def test_float64_inputs_are_computed_in_float32_and_come_back_as_given():
     with torch.no_grad():
         h, last = elementwise_recurrence_gpu(u, x, wc, bias, c0, 0, c.d, True, True)
     assert h.dtype == torch.float32
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(L=6, B=2, d=5, dirs=2, pad="right", scale=1.7, mask_c=True),
+    dict(L=5, B=2, d=3, dirs=2, k=4, act=1),
+    dict(L=4, B=2, d=3, skip=False, pad="random"),
+    dict(L=4, B=2, d=4, custom=True, act=1),
+])
+def test_gradcheck_of_the_function_in_double(cfg):
+    # finite differences of the forward kernels against the backward kernels, both in double: a check
+    # of the analytic backward pass that does not go through the oracle
+    from sru_amd import ElementwiseRecurrence
+    c = Case(seed=46, **cfg)
+    dev = "cuda:0"
+    t = lambda a: torch.tensor(a, dtype=torch.float64, device=dev, requires_grad=True)
+    u, x, wc, bias, c0 = t(c.U), t(c.x), t(c.wc), t(c.bias), t(c.c0)
+    sx = torch.tensor([c.scale], dtype=torch.float64, device=dev)
+    mc = None if c.mask_c is None else torch.tensor(c.mask_c, dtype=torch.float64, device=dev)
+    pad = None if c.pad is None else torch.tensor(c.pad, device=dev)
+    fn = lambda u, x, wc, bias, c0: ElementwiseRecurrence.apply(
+        u, x, wc, bias, c0, c.act, c.d, c.dirs == 2, c.skip_type != 0, sx, mc, pad)
+    inputs = (u, x, wc, bias, c0) if c.skip_type == 1 else (u, x.detach(), wc, bias, c0)
+    assert torch.autograd.gradcheck(fn, inputs, eps=1e-6, atol=1e-7, rtol=1e-6, nondet_tol=0.0)
 
 
 def test_no_initial_state_no_last_state_gradient_and_last_state_only():

@@ -12,6 +12,8 @@ Tolerances (the bar the build is held to):
                     max abs error <= 2e-2 * max(1, max|reference|); gradient cells
                     <= 2e-2 * max(1, |reference cell|) (per cell, so a wrong small cell cannot hide
                     behind a large one); the summed grad_wc / grad_bias <= 2e-2 * max(1, max|reference|).
+  float64 streams : everything is computed in double; the same comparisons with 1e-12 in the place
+                    of 1e-5 (the double exp of the device library against the host's).
 Outputs are pre-filled with NaN: a cell the kernels do not write fails the comparison.
 """
 import os
@@ -27,6 +29,7 @@ from tests.cases import GRID, Case
 pytestmark = pytest.mark.gpu
 
 F32_ABS = 1e-5
+F64_ABS = 1e-12
 HALF_REL = 2e-2
 
 
@@ -57,9 +60,10 @@ def check_against_oracle(case, dt="f32", keep_c=True, checkpointed=False, x_f32=
     rc = dp.rounded_case()
     h, c, c_last = dp.forward(keep_c=keep_c)
     h_ref, c_ref, cl_ref = so.forward(*rc.fwd_args(), **rc.kw())
-    tol = (lambda ref: F32_ABS) if dt == "f32" else (lambda ref: HALF_REL * _scale(ref))
+    exact = {"f32": F32_ABS, "f64": F64_ABS}.get(dt)   # absolute bar of the float and double streams
+    tol = (lambda ref: exact) if exact else (lambda ref: HALF_REL * _scale(ref))
     assert _err(to_np(h), h_ref) <= tol(h_ref)
-    assert _err(to_np(c_last), cl_ref) <= (F32_ABS if dt == "f32" else 1e-3 * _scale(cl_ref))
+    assert _err(to_np(c_last), cl_ref) <= (exact or 1e-3 * _scale(cl_ref))
     if not keep_c:
         return
     if checkpointed:
@@ -70,7 +74,7 @@ def check_against_oracle(case, dt="f32", keep_c=True, checkpointed=False, x_f32=
             s_ = (r + 1) * T - 1
             expect = np.concatenate([c_ref[s_, :, :d], c_ref[case.L - 1 - s_, :, d:]], -1) if case.dirs == 2 \
                 else c_ref[s_]
-            assert _err(to_np(c[r]), expect) <= (F32_ABS if dt == "f32" else 1e-3 * _scale(expect))
+            assert _err(to_np(c[r]), expect) <= (exact or 1e-3 * _scale(expect))
         c_used = c_ref
     else:
         assert _err(to_np(c), c_ref) <= tol(c_ref)
@@ -79,11 +83,11 @@ def check_against_oracle(case, dt="f32", keep_c=True, checkpointed=False, x_f32=
     gu, gx, gwc, gb, gi = dp.backward()
     g_ref = so.backward(*rc.fwd_args(), c_used, rc.gh, rc.gl, **rc.kw())
     # gradient cells, every stream type: error relative to max(1, |that cell|)
-    cell_tol = F32_ABS if dt == "f32" else HALF_REL
+    cell_tol = exact or HALF_REL
     assert _cell_err(to_np(gu), g_ref[0]) <= cell_tol
     if case.skip_type == 1:
         assert _cell_err(to_np(gx), g_ref[1]) <= cell_tol
-    sum_tol = (lambda ref: F32_ABS * _scale(ref)) if dt == "f32" else (lambda ref: HALF_REL * _scale(ref))
+    sum_tol = (lambda ref: (exact or HALF_REL) * _scale(ref))
     if case.custom:
         assert _cell_err(to_np(gwc), g_ref[2]) <= cell_tol
     else:
@@ -124,6 +128,19 @@ MID = [
 @pytest.mark.parametrize("cfg", MID, ids=_ids)
 def test_mid_shapes(cfg, dt):
     check_against_oracle(Case(seed=22, **cfg), dt)
+
+
+@pytest.mark.parametrize("cfg", GRID + MID, ids=_ids)
+def test_double_streams(cfg):
+    # the general kernels computing in double: streams, small tensors, state, sums
+    check_against_oracle(Case(seed=23, **cfg), "f64")
+
+
+def test_double_streams_refuse_checkpoints():
+    dp = DeviceProblem(Case(L=9, B=2, d=8, seed=1), "f64", checkpointed=True)
+    import ctypes
+    from sru_amd import _lib
+    assert _lib.load().sru_amd_state_bytes(ctypes.byref(dp.shape)) == 0   # bad flags: no size
 
 
 # every layout that can keep its state as checkpoints: all but four streams without a skip term and
