@@ -42,7 +42,7 @@ WORKLOADS = {
     "headline-infer": ("bi-SRU d=1024 L=256 B=64 k=3 forward only", 256, 64, 1024, 2, 3, True, False),
     "headline-pad": ("bi-SRU d=1024 L=256 B=64 k=3, right-padded lengths in [64,256]", 256, 64, 1024, 2, 3, False, True),
 }
-DT_BYTES = {"f32": 4, "f16": 2, "bf16": 2}
+DT_BYTES = {"f32": 4, "f16": 2, "bf16": 2, "f64": 8}
 
 
 def cpu_baseline(L, B, d, dirs, k, budget_s=12.0):
@@ -323,6 +323,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the recurrence on ONE GPU only "
                  "(columns are independent; no multi-GPU path exists): run with --gpus 1")
+    if args.dtype == "f64" and (args.workload in STACKS or args.workload == "layernorm"):
+        sys.exit("bench.py: --dtype f64 is a side measurement of the recurrence calls only (the layer stacks "
+                 "cast float64 to float32 as the reference's training entry does; layer norm has no double rows)")
     if args.workload in STACKS:
         return run_stack(args)
     if args.workload == "layernorm":
@@ -331,8 +334,8 @@ def main():
     import torch
     from sru_amd import _lib
 
-    TORCH_DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
-    CODE = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16}
+    TORCH_DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16, "f64": torch.float64}
+    CODE = {"f32": _lib.F32, "f16": _lib.F16, "bf16": _lib.BF16, "f64": _lib.F64}
 
     def p(t):   # device pointer for the C ABI
         return None if t is None else ctypes.c_void_p(t.data_ptr())
@@ -349,7 +352,10 @@ def main():
     es = DT_BYTES[args.dtype]
     lib = _lib.load()
     custom = args.per_step_weight_c
-    ckpt = not args.full_state and not fwd_only and not (args.no_skip and k == 4) and not (custom and args.tanh)
+    # (double streams: the general kernels, state after every step, small tensors in double too)
+    ckpt = not args.full_state and not fwd_only and not (args.no_skip and k == 4) and not (custom and args.tanh) \
+        and args.dtype != "f64"
+    sdt = torch.float64 if args.dtype == "f64" else torch.float32
     use_x = k == 3 and not args.no_skip      # the skip term is read from x
     if args.tanh:
         name += " tanh"
@@ -380,23 +386,23 @@ def main():
             gx=torch.empty(L, B, Dp, device=dev, dtype=xdt),
         )
         sets.append(s)
-    wc = (torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1) * 1.5 ** 0.5
+    wc = ((torch.rand(2 * Dp, device=dev, generator=g) * 2 - 1) * 1.5 ** 0.5).to(sdt)
     if custom:
         wc = (wc.view(2, Dp).t().reshape(1, 1, 2 * Dp) + 0.1 * torch.randn(L, B, 2 * Dp, device=dev, generator=g)).to(tdt)
-    bias = torch.zeros(2 * Dp, device=dev)
-    c0 = torch.zeros(B, Dp, device=dev)
-    gl = torch.zeros(B, Dp, device=dev)
-    scale = torch.tensor([3 ** 0.5], device=dev)
-    c_last = torch.empty(B, Dp, device=dev)
+    bias = torch.zeros(2 * Dp, device=dev, dtype=sdt)
+    c0 = torch.zeros(B, Dp, device=dev, dtype=sdt)
+    gl = torch.zeros(B, Dp, device=dev, dtype=sdt)
+    scale = torch.tensor([3 ** 0.5], device=dev, dtype=sdt)
+    c_last = torch.empty(B, Dp, device=dev, dtype=sdt)
     pad = None
     if padded:
         lens = torch.randint(L // 4, L + 1, (B,), device=dev, generator=g)
         if args.fixed_length:
             lens = torch.full((B,), args.fixed_length, device=dev)
         pad = (torch.arange(L, device=dev)[:, None] >= lens[None, :]).view(torch.uint8).contiguous()
-    gwc = torch.empty(L, B, 2 * Dp, device=dev, dtype=tdt) if custom else torch.empty(2 * Dp, device=dev)
-    gb = torch.empty(2 * Dp, device=dev)
-    gi = torch.empty(B, Dp, device=dev)
+    gwc = torch.empty(L, B, 2 * Dp, device=dev, dtype=tdt) if custom else torch.empty(2 * Dp, device=dev, dtype=sdt)
+    gb = torch.empty(2 * Dp, device=dev, dtype=sdt)
+    gi = torch.empty(B, Dp, device=dev, dtype=sdt)
     ws_bytes = lib.sru_amd_backward_workspace_bytes(ctypes.byref(shape))
     ws = torch.empty(ws_bytes // 4, device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
