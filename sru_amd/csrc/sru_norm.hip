@@ -231,38 +231,47 @@ layer_norm_backward(const TI *x, const float *gamma, const float *mean, const fl
     const int64_t stride = (int64_t)gridDim.x * GROUPS * R;
     Raw<TI> nx[R];
     Raw<TG> nd[R];
-    // `first` is the first row of the workgroup's trip (the same for all its groups, so that every
-    // wavefront makes the same number of trips and meets the others at the barriers); a group past
-    // the last row repeats the last row and drops it
-    int64_t first = (int64_t)blockIdx.x * GROUPS * R;
+    float nmu[R], nrs[R];
+    // The rows of a trip and their statistics are requested a trip ahead, the statistics first: a
+    // wavefront's loads return in the order they were issued, so a statistic fetched after the
+    // next trip's rows would make the current trip wait for those rows as well (44.9 -> 41.8 us at
+    // 16 384 x 2 048 in bfloat16). A group past the last row repeats the last row and drops it.
+    auto fetch = [&](int64_t row0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int64_t row = first + grp * R + r;
-        const int64_t at = (row < last ? row : last) * D;
-        nx[r].load(my_x + at);
-        nd[r].load(my_dy + at);
-    }
+        for (int r = 0; r < R; ++r) {
+            const int64_t at = row0 + r < last ? row0 + r : last;
+            nmu[r] = mean[at];
+            nrs[r] = rstd[at];
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int64_t at = (row0 + r < last ? row0 + r : last) * D;
+            nx[r].load(my_x + at);
+            nd[r].load(my_dy + at);
+        }
+    };
+    // `first` is the first row of the workgroup's trip (the same for all its groups, so that every
+    // wavefront makes the same number of trips and meets the others at the barriers)
+    int64_t first = (int64_t)blockIdx.x * GROUPS * R;
+    fetch(first + grp * R);
     int parity = 0;
     for (; first < rows; first += stride, parity ^= 1) {
         const int64_t row = first + grp * R;
-        float xh[R][kPer], gy[R][kPer], sums[2 * R], rs[R];
+        float xh[R][kPer], gy[R][kPer], sums[2 * R], rs[R], mus[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             nx[r].unpack(xh[r]);
             nd[r].unpack(gy[r]);
+            mus[r] = nmu[r];
+            rs[r] = nrs[r];
         }
-        const int64_t after = row + stride;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int64_t at = (after + r < last ? after + r : last) * D;
-            nx[r].load(my_x + at);
-            nd[r].load(my_dy + at);
-        }
+        fetch(row + stride);
+        __builtin_amdgcn_sched_barrier(0);   // the requests of the next trip go out before this trip's arithmetic
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const bool live = row + r < rows;   // a row past the end repeats the last row and is dropped
-            const float mu = live ? mean[row + r] : 0.f;
-            rs[r] = live ? rstd[row + r] : 0.f;
+            const float mu = mus[r];
+            rs[r] = live ? rs[r] : 0.f;
             float s1 = 0.f, s2 = 0.f;
             if (live) {
 #pragma unroll
