@@ -32,6 +32,9 @@ class LayerNormFunction(Function):
     @staticmethod
     def forward(ctx, x, weight, bias, eps, out_dtype):
         D = x.size(-1)
+        if weight.numel() != D or bias.numel() != D:
+            raise ValueError(f"layer norm over {D} features needs weight and bias of {D} elements, "
+                             f"not {weight.numel()} and {bias.numel()}")
         x_ = _aligned(x, 16)
         w_, b_ = _aligned(_small(weight, torch.float32), 16), _aligned(_small(bias, torch.float32), 16)
         rows = x_.numel() // D
@@ -52,7 +55,9 @@ class LayerNormFunction(Function):
         x_, w_, mean, rstd = ctx.saved_tensors
         D = x_.size(-1)
         rows = x_.numel() // D
-        gy = _aligned(grad_y, 16)
+        gy = _aligned(grad_y if grad_y.dtype in _DTYPES else grad_y.float(), 16)
+        if gy.shape != x_.shape:
+            raise ValueError(f"grad_y has shape {tuple(gy.shape)}, expected {tuple(x_.shape)}")
         grad_x = torch.empty_like(x_)
         grad_wb = torch.empty(2, D, dtype=torch.float32, device=x_.device)
         lib = _lib.load()

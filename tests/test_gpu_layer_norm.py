@@ -90,7 +90,16 @@ def test_unsupported_shapes_take_torch_layer_norm():
     with pytest.raises(ValueError, match="no kernel for"):
         layer_norm(x, w, b, strict=True)
     with pytest.raises(ValueError):
-        layer_norm(x, w, b, out_dtype=torch.float64)
+        layer_norm(torch.randn(4, 16, device=DEV), torch.randn(16, device=DEV), torch.randn(16, device=DEV),
+                   out_dtype=torch.float64)
+    # float64 rows: torch's kernel in double; parameters of the wrong size never reach a kernel
+    xd = torch.randn(4, 16, device=DEV, dtype=torch.float64)
+    wd, bd = torch.randn(16, device=DEV, dtype=torch.float64), torch.randn(16, device=DEV, dtype=torch.float64)
+    with pytest.warns(UserWarning, match="no kernel for"):
+        yd = layer_norm(xd, wd, bd)
+    assert yd.dtype == torch.float64 and torch.allclose(yd, F.layer_norm(xd, (16,), wd, bd), atol=1e-12)
+    with pytest.raises(ValueError, match="needs weight and bias"):
+        layer_norm(torch.randn(4, 16, device=DEV), torch.randn(8, device=DEV), torch.randn(16, device=DEV))
 
 
 def test_module_uses_the_kernels_and_emits_the_autocast_dtype_before_the_projection(monkeypatch):
