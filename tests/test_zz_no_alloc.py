@@ -20,9 +20,9 @@ def _static_backward(dp):
     nan = lambda *s, dtype: torch.full(s, float("nan"), dtype=dtype, device=dp.dev)
     gu = nan(c.L, c.B, c.Dp * c.k, dtype=dp.tdt)
     gx = nan(c.L, c.B, c.Dp, dtype=dp.tdt) if c.skip_type == 1 else None
-    gwc = nan(c.L, c.B, c.Dp * 2, dtype=dp.tdt) if c.custom else nan(2 * c.Dp, dtype=torch.float32)
-    gb = nan(2 * c.Dp, dtype=torch.float32)
-    gi = nan(c.B, c.Dp, dtype=torch.float32)
+    gwc = nan(c.L, c.B, c.Dp * 2, dtype=dp.tdt) if c.custom else nan(2 * c.Dp, dtype=dp.sdt)
+    gb = nan(2 * c.Dp, dtype=dp.sdt)
+    gi = nan(c.B, c.Dp, dtype=dp.sdt)
     stream = ctypes.c_void_p(torch.cuda.current_stream(dp.dev).cuda_stream)
     rc = _lib.load().sru_amd_backward_static(
         ctypes.byref(dp.shape), p(dp.U), p(dp.x) if c.skip_type == 1 else None, p(dp.wc), p(dp.bias),
@@ -32,7 +32,7 @@ def _static_backward(dp):
     return gu, gx, gwc, gb, gi
 
 
-@pytest.mark.parametrize("dt,checkpointed", [("f32", True), ("f32", False), ("bf16", True)])
+@pytest.mark.parametrize("dt,checkpointed", [("f32", True), ("f32", False), ("bf16", True), ("f64", False)])
 def test_static_backward_equals_workspace_backward_on_two_calls_in_a_row(dt, checkpointed):
     big = Case(L=40, B=16, d=256, dirs=2, seed=91, pad="right", scale=1.7, mask_c=True)
     small = Case(L=19, B=3, d=70, dirs=2, k=4, seed=92, pad="random")
@@ -68,5 +68,8 @@ def test_static_backward_rejects_more_columns_than_its_array_holds():
     too_wide = _lib.Shape(4, cols // 1024 + 1, 1024, 1, 3, 0, 1, 0, _lib.F32, 8)
     assert lib.sru_amd_backward_static(ctypes.byref(too_wide), *([fake] * 16), None) == 8
     assert "262144" in _lib.status_string(8)
+    # double partial sums fill the array with half as many columns
+    half = _lib.Shape(4, cols // 2048 + 1, 1024, 1, 3, 0, 1, 0, _lib.F64, 1)
+    assert lib.sru_amd_backward_static(ctypes.byref(half), *([fake] * 16), None) == 8
     bad = _lib.Shape(0, 1, 8, 1, 3, 0, 1, 0, _lib.F32, 8)
     assert lib.sru_amd_backward_static(ctypes.byref(bad), *([fake] * 16), None) == 2
