@@ -63,10 +63,10 @@ def _run(cmd, verbose):
     return usage
 
 
-def build(verbose=True, output=OUTPUT, defines=()):
+def build(verbose=True, output=OUTPUT, defines=(), max_scratch_bytes=MAX_SCRATCH_BYTES):
     """Compiles every translation unit (in parallel) and links the shared library.
 
-    `defines` (e.g. ["SRU_AMD_PAIR_BELOW=131072"]) and `output` serve tuning builds."""
+    `defines` (e.g. ["SRU_AMD_PAIR_BELOW=131072"]), `output` and `max_scratch_bytes` serve tuning builds."""
     from concurrent.futures import ThreadPoolExecutor
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     tag = "".join(c if c.isalnum() else "_" for c in "_".join(defines))
@@ -82,9 +82,9 @@ def build(verbose=True, output=OUTPUT, defines=()):
             usage.update(part)
     with open(os.path.join(obj_dir, "resource_usage.json"), "w") as f:
         json.dump({k: {"vgprs": v[0], "scratch_bytes": v[1]} for k, v in sorted(usage.items())}, f, indent=1)
-    spilled = {k: v[1] for k, v in usage.items() if v[1] > MAX_SCRATCH_BYTES}
+    spilled = {k: v[1] for k, v in usage.items() if v[1] > max_scratch_bytes}
     if spilled:
-        raise RuntimeError(f"{len(spilled)} kernels keep more than {MAX_SCRATCH_BYTES} bytes per lane in "
+        raise RuntimeError(f"{len(spilled)} kernels keep more than {max_scratch_bytes} bytes per lane in "
                            f"scratch memory, e.g. {sorted(spilled.items(), key=lambda kv: -kv[1])[:3]}")
     if verbose:
         print(f"{len(usage)} kernels, largest scratch {max([v[1] for v in usage.values()] or [0])} bytes/lane, "

@@ -1078,30 +1078,28 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
         typename S1::G gh[TC];
         typename SV::G w[CUSTOM ? TC : 1];
         uint32_t pad[TC];    // padding flags of the chunk's steps
-        float cstart[COLS];  // state before the chunk's first step
+        float cstart[COLS];  // state before the chunk's first step, as loaded
+        uint32_t keep;       // all ones, or zero when that state is zero whatever was loaded
     };
 
-    // n: number of valid steps in the chunk (TC except for a ragged last chunk)
-    auto load_chunk = [&](Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
-        const int64_t s0 = ch * TC;
-#pragma unroll
-        for (int i = 0; i < TC; ++i) {
-            if (i < n) {
-                const int64_t e = ef + (s0 + i) * es;
-                k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
-                if (SKIP == 1) k.x[i] = SX::template load<NTL>(xbase + e, lane, q);
-                k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
-                if constexpr (CUSTOM) k.w[i] = SV::template load<NTL>(vbase + e * 2, lane, q);
-                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
-            }
-        }
+    // Where in a chunk's burst of requests the start state goes: first, except in the builds with a
+    // padding mask (measured, kernel time: 32 768 float columns of 512 steps 125.6 us with the old
+    // placement and early mask, 116.8 us last, 108.1 us first; the same columns with 128 padded steps
+    // 33.8 / 31.0 / 33.3 us).
+    // (The two-columns-per-lane builds with per-lane row arithmetic have no register to spare for
+    // the mask: they apply it at once, as all builds did before, and request the state last.)
+    constexpr bool kLateMask = COLS == 1 || UNI;
+    constexpr bool kStartFirst = kLateMask && !HAS_PAD;
+    auto load_cstart = [&](Chunk &k, int64_t ch) __attribute__((always_inline)) {
         // one load from a selected address (a select between a register and a loaded value made the
         // compiler keep the initial state in scratch memory and select between addresses itself)
         // (without an initial state the first chunk starts from zero; its load reads checkpoint row 0,
-        // which always exists, and drops the value)
-        // (the value is dropped with a bit mask: a select makes the compiler branch around the load,
-        // inside the pipelined loop)
+        // which always exists, and the value is dropped with a bit mask when the chunk's turn comes:
+        // a select makes the compiler branch around the load, inside the pipelined loop, and a mask
+        // applied here would touch the value right after its load, which waits for it and, since a
+        // wavefront's loads return in issue order, for every load issued before it)
         const uint32_t keep = (ch == 0 && !p.c0) ? 0u : ~0u;
+        k.keep = kLateMask ? keep : ~0u;
         // The address is one of two bases. As a select it becomes a scalar branch that cuts the loop
         // body in two, which the one-column-per-lane kernels like (measured 8 % faster at 512
         // wavefronts, level at 2 048) and the two-columns-per-lane kernels do not (6 % slower at
@@ -1117,7 +1115,25 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
         }
 #pragma unroll
         for (int c = 0; c < COLS; ++c)
-            k.cstart[c] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, from[c]) & keep);
+            k.cstart[c] = kLateMask ? from[c] : __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, from[c]) & keep);
+    };
+
+    // n: number of valid steps in the chunk (TC except for a ragged last chunk)
+    auto load_chunk = [&](Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
+        const int64_t s0 = ch * TC;
+        if constexpr (kStartFirst) load_cstart(k, ch);
+#pragma unroll
+        for (int i = 0; i < TC; ++i) {
+            if (i < n) {
+                const int64_t e = ef + (s0 + i) * es;
+                k.u[i] = SU::template load<NTL>(ubase + e * K, lane, q);
+                if (SKIP == 1) k.x[i] = SX::template load<NTL>(xbase + e, lane, q);
+                k.gh[i] = S1::template load<NTL>(ghbase + e, lane, q);
+                if constexpr (CUSTOM) k.w[i] = SV::template load<NTL>(vbase + e * 2, lane, q);
+                k.pad[i] = HAS_PAD ? p.pad[pf + (s0 + i) * ps] : 0;
+            }
+        }
+        if constexpr (!kStartFirst) load_cstart(k, ch);
     };
 
     auto compute_chunk = [&](const Chunk &k, int64_t ch, int n) __attribute__((always_inline)) {
@@ -1126,7 +1142,7 @@ __global__ void __launch_bounds__(kBlock * max_waves_per_group<T>(MODE)) backwar
         float g1[TC][COLS], g2[TC][COLS];
         float u0s[TC][COLS], xs[TC][COLS];  // candidate stream and (k = 4) skip stream, decoded once
 #pragma unroll
-        for (int c = 0; c < COLS; ++c) st[0][c] = k.cstart[c];
+        for (int c = 0; c < COLS; ++c) st[0][c] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, k.cstart[c]) & k.keep);
         float gw1[COLS] = {}, gw2[COLS] = {}, gb1[COLS] = {}, gb2[COLS] = {};  // this chunk's share of the sums
 #pragma unroll
         for (int i = 0; i < TC; ++i) {

@@ -288,7 +288,9 @@ backward_scan_split(const BwdParams p) {
         typename TU::Regs u;
         typename T1::Regs x, gh;
         uint32_t pad;
-        float cstart;
+        float cstart;     // the chunk's start state as loaded; `keep` is applied when the chunk's turn comes:
+        uint32_t keep;    // touched right after its load, the value would have to arrive, and since a
+                          // wavefront's loads return in issue order, so would every tile of the chunk
     };
     int64_t ou[TU::kPieces], o1[T1::kPieces];
     TU::offsets(ou, lane, es * (K * 2));
@@ -315,8 +317,8 @@ backward_scan_split(const BwdParams p) {
         // value is dropped with a bit mask. The address stays a select: blended with bit masks like the
         // value, the loop body became one basic block and 4-5 % slower.)
         const float *from = (ch == 0) ? (p.c0 ? p.c0 + col : p.ckpt + col) : p.ckpt + (ch * kRowsPerChunk - 1) * p.ncols + col;
-        const uint32_t keep = (ch == 0 && !p.c0) ? 0u : ~0u;
-        s.cstart = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, *from) & keep);
+        s.keep = (ch == 0 && !p.c0) ? 0u : ~0u;
+        s.cstart = *from;
     };
 
     auto stage_to_lds = [&](const Stage &s) __attribute__((always_inline)) {
@@ -324,7 +326,7 @@ backward_scan_split(const BwdParams p) {
         if (SKIP == 1) T1::template to_lds<PITCH>(s.x, lds_in + TU::kRowBytes, lane);
         T1::to_lds(s.gh, lds_gh, lane);
         if (HAS_PAD) reinterpret_cast<u32_a *>(lds_pad)[lane] = s.pad;
-        lds_cstart[lane] = s.cstart;
+        lds_cstart[lane] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, s.cstart) & s.keep);
         lds_handover();
     };
 
