@@ -459,6 +459,12 @@ struct CompensatedSumOf {
 };
 using CompensatedSum = CompensatedSumOf<float>;
 
+// Waits for every vector-memory operation issued so far (s_waitcnt vmcnt(0), gfx9 encoding).
+// Placed once before a pipelined loop: whatever was loaded before the loop and is used inside it
+// would otherwise make the compiler place a wait inside the loop whose count also drains the
+// loads the loop keeps in flight on purpose.
+__device__ __forceinline__ void wait_for_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // ================================================================= forward scan
 // T: stream element type. K: streams per column in U. SKIP: 0 none, 1 from x, 2 from
 // U[..., 3]. COLS: columns per lane (2 needs an even d). P: ring depth.
@@ -912,7 +918,10 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
         s.gh = load_group<T, COLS, NTL>(ghp);
         ghp += es;
         s.first = first;
-        if (!first) s.cprev = load_group<T, COLS, NTL>(cpp);
+        // every step issues the same loads, so that the loop body stays one block and the waits count
+        // exactly: the column's first step, whose previous state is c_init and not part of the
+        // stream, reads the state after the step instead (a valid address) and drops it
+        s.cprev = load_group<T, COLS, NTL>(cpp - (es & -(int64_t)first));
         cpp += es;
         s.pad = 0;
         if (has_pad) {
@@ -973,6 +982,7 @@ __global__ void __launch_bounds__(kBlock * 4) backward_scan(const BwdParams p) {
     for (int i = 0; i < P; ++i)
         if (i < L) fetch(ring[i], i == L - 1);
 
+    wait_for_all_loads();   // the ring's first fill: the waits inside the loop then count what the loop itself issued
     int64_t s0 = 0;
     for (; s0 + 2 * P <= L; s0 += P) {
 #pragma unroll

@@ -32,12 +32,6 @@ __device__ __forceinline__ void lds_handover() {
     __builtin_amdgcn_wave_barrier();
 }
 
-// Waits for every vector-memory operation issued so far (s_waitcnt vmcnt(0), gfx9 encoding).
-// Placed once before a pipelined loop: whatever was loaded before the loop and is used inside it
-// would otherwise make the compiler place a wait inside the loop whose count also drains the
-// loads the loop keeps in flight on purpose.
-__device__ __forceinline__ void wait_for_all_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
-
 // A tile of TC rows; a row holds N 16-bit elements for each of the wavefront's W columns
 // (W = 64: one column per lane; W = 32: two lanes per column, sru_split.h).
 template <int N, int TC, int W = kBlock>
