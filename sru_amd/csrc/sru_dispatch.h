@@ -39,7 +39,10 @@ constexpr int64_t kPairBelow = SRU_AMD_PAIR_BELOW;
 
 // Lane-pair kernels (sru_split.h): 16-bit streams, d a multiple of 32, at most 1024 wavefronts of 32
 // columns, every stream 16-byte aligned, state kept as checkpoints or not at all.
-constexpr int kSplitNbuf = 2;   // chunks (of 16 steps) in flight per wavefront
+#ifndef SRU_AMD_SPLIT_NBUF   // (set by tuning builds only)
+#define SRU_AMD_SPLIT_NBUF 2
+#endif
+constexpr int kSplitNbuf = SRU_AMD_SPLIT_NBUF;   // chunks (of 16 steps) in flight per wavefront
 #ifndef SRU_AMD_SPLIT_MAX_WAVES   // (set by tuning builds only)
 #define SRU_AMD_SPLIT_MAX_WAVES 1024
 #endif
