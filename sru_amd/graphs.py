@@ -1,7 +1,7 @@
 """Replaying a stack from a HIP graph.
 
 Short sequences are bound by launches, not by kernels: the README example (2 layers, L=20, B=32,
-d=128) spends about 110 us of host time per forward around 10 us of kernels. Nothing in this
+d=128) spends about 90 us of host time per forward around 15 us of kernels. Nothing in this
 package allocates device memory behind torch's back, synchronises or reads a device value on the
 host, so a whole `SRU` forward (and backward) records into a HIP graph as it is; a replay costs one
 launch.
