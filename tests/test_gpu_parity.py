@@ -252,6 +252,7 @@ def _random_cases(n, seed):
     """Seeded draw over everything the boundary accepts: sizes around the wavefront, pair and
     chunk boundaries, both directions, every flag combination the shape check allows."""
     rng = np.random.default_rng(seed)
+    to_double = np.random.default_rng(seed + 1)   # (its own stream: the other draws stay what they were)
     out = []
     for i in range(n):
         k = int(rng.choice([3, 4]))
@@ -266,7 +267,10 @@ def _random_cases(n, seed):
                    scale=float(rng.choice([1.0, 0.6, 1.7])) if (k == 3 and skip) else None,
                    zero_c0=bool(rng.random() < 0.3))
         dt = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
-        out.append((cfg, dt, bool(rng.random() < 0.5), 1000 + i))
+        ckpt = bool(rng.random() < 0.5)
+        if to_double.random() < 0.15:     # double streams: state after every step only
+            dt, ckpt = "f64", False
+        out.append((cfg, dt, ckpt, 1000 + i))
     return out
 
 
