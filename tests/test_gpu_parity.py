@@ -136,6 +136,15 @@ def test_double_streams(cfg):
     check_against_oracle(Case(seed=23, **cfg), "f64")
 
 
+def test_double_streams_without_state_store():
+    # the inference variant (c == NULL) of the double kernels: same h and last state, bit for bit
+    c = Case(L=19, B=3, d=70, dirs=2, seed=27, pad="right", scale=1.3, mask_c=True)
+    dp = DeviceProblem(c, "f64")
+    h, _, c_last = [t.clone() if t is not None else None for t in dp.forward(keep_c=True)]
+    h2, none, c_last2 = dp.forward(keep_c=False)
+    assert none is None and torch.equal(h, h2) and torch.equal(c_last, c_last2)
+
+
 def test_double_streams_refuse_checkpoints():
     dp = DeviceProblem(Case(L=9, B=2, d=8, seed=1), "f64", checkpointed=True)
     import ctypes
